@@ -1,0 +1,160 @@
+"""Benchmark of the PAM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = the six PAM matrix products of a DeiT-tiny MLP block on 64 x 197 tokens
+(fp32, synthetic data): for each of the layers 192->768 and 768->192 the forward product,
+dX and dW (the approximate backward of the reference's training recipe,
+pam/cuda_bindings.py:154-161).  `value` is G PAM-MAC/s over whole steps with all operands
+resident in HBM.  Each product is also timed on its own with HIP events, which gives the
+roofline figure of the matrix kernel (VALU issue rate: 2 lane-ops per MAC against
+CUs x 64 lanes x clock), and the elementwise multiply / divide are timed on 2^26
+elements against HBM bandwidth.  The CPU baseline is this repository's own C restatement
+of the same arithmetic (oracle/, OpenMP) on the host cores, on the 192->768 layer.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-elementwise", action="store_true")
+    return ap.parse_args()
+
+
+def event_time_ms(fn, iters, torch):
+    """Average duration of fn() over `iters` back-to-back launches, HIP events on the launch stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fn(); torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
+                 "(the path has no collective; see DESIGN.md for how it would shard)")
+    import torch
+    from pam_amd import _abi
+    from pam_amd._abi import HipKernels
+    _abi.load_library()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    K = HipKernels()
+    dev = torch.device("cuda:0")
+    cus, khz = _abi.device_info()
+    lane_peak = cus * 64 * khz * 1e3                      # VALU lane-ops per second
+
+    g = torch.Generator(device="cpu").manual_seed(0)
+    T, D1, D2 = 64 * 197, 192, 768
+    X1 = torch.randn(T, D1, generator=g).to(dev)
+    X2 = torch.randn(T, D2, generator=g).to(dev)
+    W1 = torch.nn.init.trunc_normal_(torch.empty(D2, D1), std=0.02, a=-0.04, b=0.04, generator=g).to(dev)
+    W2 = torch.nn.init.trunc_normal_(torch.empty(D1, D2), std=0.02, a=-0.04, b=0.04, generator=g).to(dev)
+    dY1 = (torch.randn(T, D2, generator=g) * 1e-2).to(dev)
+    dY2 = (torch.randn(T, D1, generator=g) * 1e-2).to(dev)
+
+    products = {
+        "fwd_12608x768x192": lambda: K.pam_matmul_fwd(X1, W1.T, True, False, 1.0),
+        "dX_12608x192x768": lambda: K.pam_matmul_fwd(dY1, W1, True, True, 1.0),
+        "dW_192x768x12608": lambda: K.pam_matmul_fwd(X1.T, dY1, False, True, 1.0),
+        "fwd_12608x192x768": lambda: K.pam_matmul_fwd(X2, W2.T, True, False, 1.0),
+        "dX_12608x768x192": lambda: K.pam_matmul_fwd(dY2, W2, True, True, 1.0),
+        "dW_768x192x12608": lambda: K.pam_matmul_fwd(X2.T, dY2, False, True, 1.0),
+    }
+    macs_each = T * D1 * D2
+
+    def step():
+        for fn in products.values():
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    gmacs = len(products) * macs_each / (dt / args.steps) / 1e9
+
+    per = {}
+    for name, fn in products.items():
+        ms = event_time_ms(fn, max(10, args.steps), torch)
+        per[name] = {"ms": round(ms, 4), "gmacs": round(macs_each / ms / 1e6, 1),
+                     "valu_frac": round(2 * macs_each / (ms * 1e-3) / lane_peak, 4)}
+    head = per["fwd_12608x768x192"]
+    roofline = {
+        "kernel": "gemm_kernel (PAM forward, 12608x768x192)", "bound": "valu",
+        "achieved": round(2 * macs_each / (head["ms"] * 1e-3) / 1e12, 3),
+        "peak": round(lane_peak / 1e12, 3), "unit": "Tlaneop/s",
+        "frac": head["valu_frac"], "traffic": None,
+        "note": "2 VALU lane-ops (v_add_u32 + v_add_f32) per PAM-MAC; peak = CUs x 64 lanes x clock; "
+                "MFMA does not apply to an integer-add product",
+        "compute_units": cus, "clock_mhz": khz / 1e3,
+        "worst_of_six_frac": min(p["valu_frac"] for p in per.values()),
+    }
+
+    out = {
+        "metric": "pam_gemm_throughput", "value": round(gmacs, 1), "unit": "GMAC/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "DeiT-tiny PAM linear fwd+dX+dW, tokens 64x197=12608, 192->768 and 768->192 "
+                               "(BASELINE configs[2]); 6 products of 1 859 125 248 PAM-MAC per step"},
+        "roofline": roofline, "products": per,
+    }
+
+    if not args.no_elementwise:
+        n = 1 << 26
+        a = torch.randn(n, generator=g).to(dev); b = torch.randn(n, generator=g).to(dev)
+        idx = torch.randint(0, n, (n // 50,), generator=g).to(dev)         # 2 % edge values
+        edge = torch.tensor([0.0, -0.0, float("inf"), float("nan"), 1e-40, -1e-41, 3e38, -2.5e38], device=dev)
+        a[idx] = edge[torch.arange(idx.numel(), device=dev) % 8]
+        b[idx.flip(0)] = edge[(torch.arange(idx.numel(), device=dev) + 3) % 8]
+        ew = {}
+        for name, fn in (("mul", lambda: K.pam_fwd(a, b, 1.0)), ("div", lambda: K.pad_fwd(a, b, 1.0))):
+            ms = event_time_ms(fn, 20, torch)
+            ew[name] = {"ms": round(ms, 4), "GBps": round(12 * n / ms / 1e6, 1)}
+        out["roofline_elementwise"] = {
+            "kernel": "ew_vec_kernel (PAM multiply, 2^26 elements, BASELINE configs[1])", "bound": "hbm",
+            "achieved": ew["mul"]["GBps"], "peak": 8000.0, "unit": "GB/s", "frac": round(ew["mul"]["GBps"] / 8000.0, 4),
+            "traffic": None, "bytes_per_element": 12, "div_GBps": ew["div"]["GBps"],
+        }
+        del a, b
+
+    if not args.no_cpu_baseline:
+        from oracle import pam_oracle as oracle
+        oracle.build()
+        cores = len(os.sched_getaffinity(0))
+        os.environ.setdefault("OMP_NUM_THREADS", str(cores))
+        Xh, Wh, dYh = X1.cpu().numpy(), W1.cpu().numpy(), dY1.cpu().numpy()
+        WT = np.ascontiguousarray(Wh.T); XT = np.ascontiguousarray(Xh.T)
+        t0 = time.perf_counter()
+        oracle.gemm_fast(Xh, WT); oracle.gemm_fast(dYh, Wh); oracle.gemm_fast(XT, dYh)
+        cdt = time.perf_counter() - t0
+        out["cpu_baseline"] = {
+            "value": round(3 * macs_each / cdt / 1e9, 2), "unit": "GMAC/s", "cores": int(os.environ.get("OMP_NUM_THREADS", cores)),
+            "kind": "port",
+            "sample": "fwd + dX + dW of the 192->768 layer once (5.58 G PAM-MAC), this repository's C restatement "
+                      "(integer add + fp32 accumulate, OpenMP over rows), contiguous operands",
+        }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,118 @@
+/*
+ * pam_hip.h -- C ABI of libpam_hip.so, the MI355X (gfx950) implementation of the
+ * piecewise-affine arithmetic kernels of epfml/pam.
+ *
+ * The fourteen compute entry points are the fourteen functions of the reference's
+ * extension module (PYBIND11_MODULE in pam/cuda_kernels.cu:932-947), one to one and under
+ * the same names with a pam_hip_ prefix.  Where the reference takes torch tensors and
+ * returns a new one, these take raw device pointers plus sizes and element strides and
+ * write into a caller-provided output.
+ *
+ * Conventions
+ *   - every pointer is a device pointer to fp32 data on the current HIP device;
+ *   - `offset` is the PAM offset as a float, 1.0f meaning none (the reference maps
+ *     offset=None to 1.0, pam/cuda_bindings.py:31-32, and turns it into a bit-pattern
+ *     increment, pam/cuda_kernels.cu:168);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls only
+ *     enqueue work, they never synchronise, allocate or free;
+ *   - return value 0 on success, negative on error; pam_hip_last_error() then returns a
+ *     message for the calling thread.  Nothing is thrown.
+ *   - matrices are described by (rows, cols) and element strides; any strides are
+ *     accepted, and the fast paths apply when one of the two strides of an operand is 1
+ *     (the row-major / column-major flags of the reference, pam/cuda_bindings.py:106-115).
+ */
+#ifndef PAM_HIP_H
+#define PAM_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PAM_HIP_ABI_VERSION 1
+
+enum {
+    PAM_HIP_OK = 0,
+    PAM_HIP_ERR_ARGUMENT = -1,   /* null pointer, negative size, size beyond 2^31 elements per dim */
+    PAM_HIP_ERR_LAUNCH = -2,     /* the HIP runtime reported an error at launch */
+    PAM_HIP_ERR_WORKSPACE = -3   /* workspace given but smaller than pam_hip_gemm_workspace_bytes() */
+};
+
+int pam_hip_abi_version(void);
+const char *pam_hip_last_error(void);
+
+/* Compute units and shader clock (kHz) of the current device, for roofline figures. */
+int pam_hip_device_info(int *compute_units, int *clock_khz);
+
+/* ---- elementwise, n contiguous elements (pam/cuda_kernels.cu:141-328) ------------------ */
+/* C = A (*) B                         replaces pam_fwd  (elementwise_pam_caller,  :155-183) */
+int pam_hip_pam_fwd(const float *a, const float *b, float *c, size_t n, float offset, void *stream);
+/* dA = d/dA (A (*) B) * dC, exact     replaces pam_bwd  (elementwise_pam_bwd_caller, :200-232) */
+int pam_hip_pam_bwd(const float *a, const float *b, const float *dc, float *da, size_t n, float offset, void *stream);
+/* C = A (/) B                         replaces pad_fwd  (elementwise_pad_caller,  :251-279) */
+int pam_hip_pad_fwd(const float *a, const float *b, float *c, size_t n, float offset, void *stream);
+/* dB = d/dB (A (/) B) * dC            replaces pad_bwd  (elementwise_pad_bwd_caller, :296-328) */
+int pam_hip_pad_bwd(const float *a, const float *b, const float *dc, float *db, size_t n, float offset, void *stream);
+
+/* Variants of the two forward ops with one operand a single fp32 value in device memory
+ * (the reference materialises broadcast scalars with flatten(), pam/cuda_kernels.cu:163-164;
+ * these read 8 B/element instead of 12).  scalar_is_a != 0: C = s[0] (op) X, else C = X (op) s[0]. */
+int pam_hip_pam_fwd_bcast(const float *x, const float *s, int scalar_is_a, float *c, size_t n, float offset, void *stream);
+int pam_hip_pad_fwd_bcast(const float *x, const float *s, int scalar_is_a, float *c, size_t n, float offset, void *stream);
+
+/* ---- piecewise-affine exp / log (pam/cuda_kernels.cu:334-516) -------------------------- */
+/* Y = base^X  = pa_exp2(X (*) log2 base)        replaces pa_exp_fwd (:348-373) */
+int pam_hip_pa_exp_fwd(const float *x, float *y, size_t n, float base, float offset, void *stream);
+/*                                                replaces pa_exp_bwd (:395-423) */
+int pam_hip_pa_exp_bwd(const float *x, const float *dy, float *dx, size_t n, float base, float offset, void *stream);
+/* Y = log_base X = pa_log2(X) (/) log2 base     replaces pa_log_fwd (:443-468) */
+int pam_hip_pa_log_fwd(const float *x, float *y, size_t n, float base, float offset, void *stream);
+/*                                                replaces pa_log_bwd (:488-516) */
+int pam_hip_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, float base, float offset, void *stream);
+
+/* ---- matrix products (pam/cuda_kernels.cu:574-927) ------------------------------------- */
+/* A matrix operand: pointer, batch stride, row stride, column stride (elements). */
+#define PAM_HIP_MAT(name) const float *name, long name##_sb, long name##_sr, long name##_sc
+#define PAM_HIP_OUT(name) float *name, long name##_sb, long name##_sr, long name##_sc
+
+/* Scratch needed by the split-K path that large-K, small-output products use (0 if the
+ * shape does not use it).  Passing workspace == NULL to the calls below is always valid
+ * and simply disables that path. */
+size_t pam_hip_gemm_workspace_bytes(long batch, long m, long n, long k);
+
+/* The accumulation order a product of this shape uses when the workspace is supplied:
+ * *k_chunk consecutive k are summed in ascending order from +0 into one accumulator per
+ * output; with *k_splits > 1 the chunk sums are then added in ascending chunk order, again
+ * from +0.  Without a workspace the order is always one chunk (plain ascending k), which is
+ * the order of the reference kernel (pam/cuda_kernels.cu:601, 608-627). */
+int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_splits, int *k_chunk);
+
+/* Y[m,n] = sum_k A[m,k] (*) B[k,n]            replaces pam_matmul_fwd (matmul_caller<&pam,false>, :703-718) */
+int pam_hip_pam_matmul_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
+                           float *y, long y_sr, long y_sc, long m, long n, long k, float offset,
+                           void *workspace, size_t workspace_bytes, void *stream);
+/* batched                                     replaces pam_bmm_fwd (matmul_caller<&pam,true>) */
+int pam_hip_pam_bmm_fwd(PAM_HIP_MAT(a), PAM_HIP_MAT(b), PAM_HIP_OUT(y), long batch, long m, long n, long k,
+                        float offset, void *workspace, size_t workspace_bytes, void *stream);
+/* ordinary fp32 multiply through the same kernel   replaces standard_matmul / standard_bmm (:941-942) */
+int pam_hip_standard_matmul(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
+                            float *y, long y_sr, long y_sc, long m, long n, long k, float ignored,
+                            void *workspace, size_t workspace_bytes, void *stream);
+int pam_hip_standard_bmm(PAM_HIP_MAT(a), PAM_HIP_MAT(b), PAM_HIP_OUT(y), long batch, long m, long n, long k,
+                         float ignored, void *workspace, size_t workspace_bytes, void *stream);
+/* Exact backward: dM[i,j] = sum_k pam_bwd(M[i,j], other, delta), where delta_l != 0 means
+ * L[i,k] is the upstream gradient and R[k,j] the other forward operand, and delta_l == 0
+ * the reverse.          replaces pam_matmul_bwd / pam_bmm_bwd (pam_matmul_bwd_caller, :894-924) */
+int pam_hip_pam_matmul_bwd(const float *l, long l_sr, long l_sc, const float *r, long r_sr, long r_sc,
+                           const float *mo, long mo_sr, long mo_sc, float *dm, long dm_sr, long dm_sc,
+                           long m, long n, long k, int delta_l, float offset,
+                           void *workspace, size_t workspace_bytes, void *stream);
+int pam_hip_pam_bmm_bwd(PAM_HIP_MAT(l), PAM_HIP_MAT(r), PAM_HIP_MAT(mo), PAM_HIP_OUT(dm),
+                        long batch, long m, long n, long k, int delta_l, float offset,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PAM_HIP_H */

@@ -330,7 +330,8 @@ void pamo_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, float
  *
  * mode 0  PAM forward; the offset is folded into the right operand first,
  *         R' = pam(R, offset), so each product is pam(L, R')
- * mode 1  ordinary fp32 multiply (standard_mul, pam/cuda_kernels.cu:522-524)
+ * mode 1  ordinary fp32 multiply (standard_mul, pam/cuda_kernels.cu:522-524), fused into the
+ *         accumulate as one fma, which is what the reference's compiler does with a*b + c
  * mode 2  exact backward, delta on the left:  pam_bwd(D[i][j], R[k][j], L[i][k])
  * mode 3  exact backward, delta on the right: pam_bwd(D[i][j], L[i][k], R[k][j])
  *         (operand roles pam/cuda_kernels.cu:795-809)
@@ -364,7 +365,7 @@ void pamo_gemm(int mode, long batch, long M, long N, long K,
                         float l = Lp[k * lc], r = Rp[k * rr], p;
                         switch (mode) {
                         case 0: p = pam1(l, off == 1.0f ? r : pam1(r, off)); break;
-                        case 1: p = l * r; break;
+                        case 1: acc = fmaf(l, r, acc); continue;   /* nvcc contracts a*b + c into one fma */
                         case 2: p = pam_bwd1(d, r, l, off); break;
                         default: p = pam_bwd1(d, l, r, off); break;
                         }

@@ -1,0 +1,254 @@
+"""ctypes binding of libpam_hip.so and the tensor-level kernel object built on it.
+
+`HipKernels` exposes the fourteen functions of the reference's extension module
+(pam/cuda_kernels.cu:932-947) with the same names, argument order and return convention
+(a new tensor; inputs untouched).  PyTorch is used for device memory and the current
+stream only.  There is no CPU fallback: a missing library or a non-GPU tensor raises.
+"""
+import ctypes
+import pathlib
+
+import torch
+
+_LIB_PATH = pathlib.Path(__file__).resolve().parent / "lib" / "libpam_hip.so"
+
+_f = ctypes.c_float
+_p = ctypes.c_void_p
+_l = ctypes.c_long
+_z = ctypes.c_size_t
+_i = ctypes.c_int
+
+_MAT = [_p, _l, _l, _l]          # pointer, batch stride, row stride, col stride
+_MAT2 = [_p, _l, _l]             # pointer, row stride, col stride
+
+_SIGNATURES = {
+    "pam_hip_abi_version": ([], _i),
+    "pam_hip_last_error": ([], ctypes.c_char_p),
+    "pam_hip_device_info": ([ctypes.POINTER(_i), ctypes.POINTER(_i)], _i),
+    "pam_hip_pam_fwd": ([_p, _p, _p, _z, _f, _p], _i),
+    "pam_hip_pam_bwd": ([_p, _p, _p, _p, _z, _f, _p], _i),
+    "pam_hip_pad_fwd": ([_p, _p, _p, _z, _f, _p], _i),
+    "pam_hip_pad_bwd": ([_p, _p, _p, _p, _z, _f, _p], _i),
+    "pam_hip_pam_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
+    "pam_hip_pad_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
+    "pam_hip_pa_exp_fwd": ([_p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_pa_exp_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_pa_log_fwd": ([_p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_pa_log_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_gemm_workspace_bytes": ([_l, _l, _l, _l], _z),
+    "pam_hip_gemm_plan": ([_l, _l, _l, _l, ctypes.POINTER(_i), ctypes.POINTER(_i)], _i),
+    "pam_hip_pam_matmul_fwd": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_pam_bmm_fwd": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_standard_matmul": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_standard_bmm": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_pam_matmul_bwd": (_MAT2 * 4 + [_l, _l, _l, _i, _f, _p, _z, _p], _i),
+    "pam_hip_pam_bmm_bwd": (_MAT * 4 + [_l, _l, _l, _l, _i, _f, _p, _z, _p], _i),
+}
+
+_lib = None
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def load_library():
+    """Loads libpam_hip.so; raises if it has not been built (python -m pam_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build the HIP extension first (python -m pam_amd.build). "
+                "This package has no CPU or PyTorch fallback.")
+        lib = ctypes.CDLL(str(_LIB_PATH))
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        if lib.pam_hip_abi_version() != 1:
+            raise RuntimeError("libpam_hip.so has an unexpected ABI version")
+        _lib = lib
+    return _lib
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES)
+
+
+def _call(name, *args):
+    lib = load_library()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        msg = lib.pam_hip_last_error().decode(errors="replace")
+        raise (ValueError if rc == -1 else RuntimeError)(f"{name} failed ({rc}): {msg}")
+
+
+def device_info():
+    cu, khz = _i(0), _i(0)
+    _call("pam_hip_device_info", ctypes.byref(cu), ctypes.byref(khz))
+    return cu.value, khz.value
+
+
+def gemm_plan(batch, m, n, k):
+    """(k_splits, k_chunk): the accumulation order used for this shape."""
+    s, c = _i(0), _i(0)
+    _call("pam_hip_gemm_plan", batch, m, n, k, ctypes.byref(s), ctypes.byref(c))
+    return s.value, c.value
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(*tensors):
+    for t in tensors:
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise RuntimeError("argument must be a CUDA tensor")      # CHECK_CUDA, pam/cuda_kernels.cu:8
+        if t.dtype != torch.float32:
+            raise TypeError(f"PAM kernels compute in float32, got {t.dtype}")
+
+
+def _is_single_value(t):
+    return t.numel() > 1 and all(s == 0 for s in t.stride())
+
+
+def _flat(t):
+    """Contiguous 1-D view; copies only when the tensor is not already contiguous
+    (the reference's flatten(), pam/cuda_kernels.cu:163-165)."""
+    return t.contiguous().view(-1)
+
+
+class HipKernels:
+    """The kernel object the autograd layer calls; same surface as the reference's
+    `cuda_kernels` extension module."""
+
+    # ---------------------------------------------------------------- elementwise
+    @staticmethod
+    def _binary(name, A, B, offset):
+        _check(A, B)
+        if A.shape != B.shape:
+            raise ValueError(f"{name}: operands must have the same shape, got {tuple(A.shape)} and {tuple(B.shape)}")
+        out = torch.empty(A.shape, dtype=torch.float32, device=A.device)
+        n = out.numel()
+        if n == 0:
+            return out
+        with torch.cuda.device(A.device):
+            if name in ("pam_fwd", "pad_fwd") and (_is_single_value(A) or _is_single_value(B)):
+                scalar_is_a = _is_single_value(A)
+                s, x = (A, B) if scalar_is_a else (B, A)
+                if _is_single_value(x):
+                    x = x.contiguous()
+                x = _flat(x)
+                _call(f"pam_hip_{name}_bcast", x.data_ptr(), s.data_ptr(), int(scalar_is_a), out.data_ptr(), n,
+                      float(offset), _stream())
+            else:
+                a, b = _flat(A), _flat(B)
+                _call(f"pam_hip_{name}", a.data_ptr(), b.data_ptr(), out.data_ptr(), n, float(offset), _stream())
+        return out
+
+    @staticmethod
+    def _ternary(name, A, B, dC, offset):
+        _check(A, B, dC)
+        if not (A.shape == B.shape == dC.shape):
+            raise ValueError(f"{name}: operands must have the same shape")
+        out = torch.empty(A.shape, dtype=torch.float32, device=A.device)
+        n = out.numel()
+        if n:
+            a, b, d = _flat(A), _flat(B), _flat(dC)
+            with torch.cuda.device(A.device):
+                _call(f"pam_hip_{name}", a.data_ptr(), b.data_ptr(), d.data_ptr(), out.data_ptr(), n, float(offset), _stream())
+        return out
+
+    def pam_fwd(self, A, B, offset):
+        return self._binary("pam_fwd", A, B, offset)
+
+    def pad_fwd(self, A, B, offset):
+        return self._binary("pad_fwd", A, B, offset)
+
+    def pam_bwd(self, A, B, dC, offset):
+        return self._ternary("pam_bwd", A, B, dC, offset)
+
+    def pad_bwd(self, A, B, dC, offset):
+        return self._ternary("pad_bwd", A, B, dC, offset)
+
+    # ---------------------------------------------------------------- exp / log
+    @staticmethod
+    def _unary(name, X, base, offset, dY=None):
+        _check(X) if dY is None else _check(X, dY)
+        out = torch.empty(X.shape, dtype=torch.float32, device=X.device)
+        n = out.numel()
+        if n:
+            x = _flat(X)
+            with torch.cuda.device(X.device):
+                if dY is None:
+                    _call(f"pam_hip_{name}", x.data_ptr(), out.data_ptr(), n, float(base), float(offset), _stream())
+                else:
+                    d = _flat(dY)
+                    _call(f"pam_hip_{name}", x.data_ptr(), d.data_ptr(), out.data_ptr(), n, float(base), float(offset), _stream())
+        return out
+
+    def pa_exp_fwd(self, X, base, offset):
+        return self._unary("pa_exp_fwd", X, base, offset)
+
+    def pa_log_fwd(self, X, base, offset):
+        return self._unary("pa_log_fwd", X, base, offset)
+
+    def pa_exp_bwd(self, X, dY, base, offset):
+        return self._unary("pa_exp_bwd", X, base, offset, dY)
+
+    def pa_log_bwd(self, X, dY, base, offset):
+        return self._unary("pa_log_bwd", X, base, offset, dY)
+
+    # ---------------------------------------------------------------- matrix products
+    @staticmethod
+    def _mat(t, batched):
+        s = t.stride()
+        return (t.data_ptr(), s[0], s[1], s[2]) if batched else (t.data_ptr(), s[0], s[1])
+
+    @classmethod
+    def _product(cls, name, batched, L, R, Mop, extra, offset):
+        ops = (L, R) if Mop is None else (L, R, Mop)
+        _check(*ops)
+        nd = 3 if batched else 2
+        if any(t.dim() != nd for t in ops):
+            raise ValueError(f"{name}: expected {nd}-D operands")
+        if L.shape[-1] != R.shape[-2] or (batched and L.shape[0] != R.shape[0]):
+            raise ValueError(f"{name}: shapes {tuple(L.shape)} and {tuple(R.shape)} do not multiply")
+        batch = L.shape[0] if batched else 1
+        m, k, n = L.shape[-2], L.shape[-1], R.shape[-1]
+        if Mop is not None and tuple(Mop.shape[-2:]) != (m, n):
+            raise ValueError(f"{name}: third operand must have the shape of the result")
+        out = torch.empty((batch, m, n) if batched else (m, n), dtype=torch.float32, device=L.device)
+        if out.numel() == 0:
+            return out
+        with torch.cuda.device(L.device):
+            lib = load_library()
+            ws_bytes = lib.pam_hip_gemm_workspace_bytes(batch, m, n, k)
+            ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=L.device) if ws_bytes else None
+            args = []
+            for t in ops:
+                args += cls._mat(t, batched)
+            args += cls._mat(out, batched)
+            args += ([batch] if batched else []) + [m, n, k] + extra + [float(offset)]
+            args += [ws.data_ptr() if ws is not None else None, ws_bytes, _stream()]
+            _call(f"pam_hip_{name}", *args)
+        return out
+
+    def pam_matmul_fwd(self, A, B, A_row_major, B_row_major, offset):
+        # the layout flags of the reference select a kernel instance there; here the strides do
+        return self._product("pam_matmul_fwd", False, A, B, None, [], offset)
+
+    def pam_bmm_fwd(self, A, B, A_row_major, B_row_major, offset):
+        return self._product("pam_bmm_fwd", True, A, B, None, [], offset)
+
+    def standard_matmul(self, A, B, A_row_major, B_row_major, offset):
+        return self._product("standard_matmul", False, A, B, None, [], offset)
+
+    def standard_bmm(self, A, B, A_row_major, B_row_major, offset):
+        return self._product("standard_bmm", True, A, B, None, [], offset)
+
+    def pam_matmul_bwd(self, L, R, M, L_row_major, R_row_major, delta_L, offset):
+        return self._product("pam_matmul_bwd", False, L, R, M, [int(bool(delta_L))], offset)
+
+    def pam_bmm_bwd(self, L, R, M, L_row_major, R_row_major, delta_L, offset):
+        return self._product("pam_bmm_bwd", True, L, R, M, [int(bool(delta_L))], offset)

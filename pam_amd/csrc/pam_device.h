@@ -1,0 +1,200 @@
+// Scalar piecewise-affine arithmetic for gfx950 device code.
+//
+// Every function takes and returns fp32 values; "bits" are their IEEE-754 patterns.
+// The common case (normal operands, normal result) is the integer add of the
+// reference's GPU kernel (pam/cuda_kernels.cu:17-19, 62-64).  Everything that kernel
+// delegates to a float-multiply guard is decided here on the bit patterns instead, and
+// follows the classes of the reference's float emulation (pam/native.py:16-20, 38-39,
+// 54-55, 163-164): inf/NaN operands give NaN, a zero operand gives a zero whose sign is
+// that of the other operand, subnormal operands count as the real numbers they are,
+// results underflow gradually (round to nearest even) and overflow to +-inf.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pamdev {
+
+constexpr uint32_t kBias = 0x3f800000u;
+constexpr uint32_t kMant = 0x007fffffu;
+constexpr uint32_t kExpo = 0x7f800000u;
+constexpr uint32_t kSign = 0x80000000u;
+constexpr uint32_t kQNaN = 0x7fc00000u;
+
+__device__ __forceinline__ uint32_t f2u(float x) { return __float_as_uint(x); }
+__device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
+
+// Finite non-zero magnitude -> unbiased exponent and 23-bit fraction, subnormals normalised.
+__device__ __forceinline__ void split_mag(uint32_t mag, int& e, uint32_t& m)
+{
+    if (mag >= 0x00800000u) { e = (int)(mag >> 23) - 127; m = mag & kMant; }
+    else {
+        int sh = __clz((int)mag) - 8;            // brings the leading one to bit 23
+        e = -126 - sh; m = (mag << sh) & kMant;
+    }
+}
+
+// sign | 2^E (1 + M / 2^23) rounded once (nearest even) into fp32; E >= 128 -> inf,
+// E <= -150 -> 0 (the reference evaluates 2**E first, and 2**-150 is already 0).
+__device__ __forceinline__ uint32_t join_mag(uint32_t sign, int E, uint32_t M)
+{
+    if (E >= 128) return sign | kExpo;
+    if (E <= -150) return sign;
+    if (E >= -126) return sign | ((uint32_t)(E + 127) << 23) | M;
+    uint32_t sig = 0x00800000u | M;
+    int sh = -126 - E;                           // 1 .. 23
+    uint32_t q = sig >> sh;
+    uint32_t rest = sig << (32 - sh);            // discarded bits, left aligned
+    q += (rest > 0x80000000u) || (rest == 0x80000000u && (q & 1u));
+    return sign | q;
+}
+
+__device__ __noinline__ float pam_general(uint32_t ai, uint32_t bi)
+{
+    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
+    if (ma >= kExpo || mb >= kExpo) return u2f(kQNaN);
+    if (ma == 0 || mb == 0) {
+        uint32_t s = (ma ? ai : 0u) ^ (mb ? bi : 0u);
+        return u2f(s & kSign);
+    }
+    int ea, eb; uint32_t fa, fb;
+    split_mag(ma, ea, fa); split_mag(mb, eb, fb);
+    uint32_t M = fa + fb; int E = ea + eb;
+    if (M & 0x00800000u) { E += 1; M &= kMant; }
+    return u2f(join_mag((ai ^ bi) & kSign, E, M));
+}
+
+// PAM product a (*) b.
+__device__ __forceinline__ float pam_mul(float a, float b)
+{
+    uint32_t ai = f2u(a), bi = f2u(b);
+    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
+    uint32_t s = ma + mb - kBias;                // magnitude of the product when all is normal
+    bool normal = (ma - 0x00800000u < 0x7f000000u) & (mb - 0x00800000u < 0x7f000000u) &
+                  (s - 0x00800000u < 0x7f000000u);
+    if (__builtin_expect(normal, 1)) return u2f(s | ((ai ^ bi) & kSign));
+    return pam_general(ai, bi);
+}
+
+__device__ __noinline__ float pad_general(uint32_t ai, uint32_t bi)
+{
+    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
+    if (ma >= kExpo || mb >= kExpo) return u2f(kQNaN);
+    if (mb == 0) return u2f(ma == 0 ? kQNaN : ((ai & kSign) | kExpo));
+    if (ma == 0) return u2f(bi & kSign);
+    int ea, eb; uint32_t fa, fb;
+    split_mag(ma, ea, fa); split_mag(mb, eb, fb);
+    int E = ea - eb; uint32_t M = fa - fb;
+    if (M & kSign) { E -= 1; M += 0x00800000u; }
+    return u2f(join_mag((ai ^ bi) & kSign, E, M));
+}
+
+// PAM quotient a (/) b.
+__device__ __forceinline__ float pad_div(float a, float b)
+{
+    uint32_t ai = f2u(a), bi = f2u(b);
+    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
+    uint32_t s = ma - mb + kBias;
+    bool normal = (ma - 0x00800000u < 0x7f000000u) & (mb - 0x00800000u < 0x7f000000u) &
+                  (s - 0x00800000u < 0x7f000000u);
+    if (__builtin_expect(normal, 1)) return u2f(s | ((ai ^ bi) & kSign));
+    return pad_general(ai, bi);
+}
+
+// The offset is one more PAM product (quotient for pad) applied to the result
+// (pam/native.py:59-60, 168-169); 1.0 switches it off (pam/cuda_bindings.py:31-32).
+__device__ __forceinline__ float pam_mul_off(float a, float b, float off, bool has_off)
+{ float c = pam_mul(a, b); return has_off ? pam_mul(c, off) : c; }
+__device__ __forceinline__ float pad_div_off(float a, float b, float off, bool has_off)
+{ float c = pad_div(a, b); return has_off ? pad_div(c, off) : c; }
+
+// 2**k for an integer k the way fp32 pow gives it: exact down to 2^-149, 0 below, inf above 127.
+__device__ __forceinline__ float pow2_int(int k)
+{
+    uint32_t u = k >= 128 ? kExpo : k >= -126 ? (uint32_t)(k + 127) << 23 : k >= -149 ? 1u << (k + 149) : 0u;
+    return u2f(u);
+}
+
+// pa_log2 (pam/native.py:24-30): exponent plus mantissa fraction of |x|, one rounding.
+__device__ __forceinline__ float pa_log2(float x)
+{
+    uint32_t mag = f2u(x) & ~kSign;
+    if (mag >= kExpo) return u2f(kQNaN);
+    if (mag == 0) return u2f(0xff800000u);
+    int e; uint32_t m; split_mag(mag, e, m);
+    return (float)(e * (1 << 23) + (int)m) * 0x1p-23f;
+}
+
+// pa_exp2 (pam/native.py:34-39): 2**floor(x) * ((1 + x) - floor(x)), fp32 operations in that order.
+__device__ __forceinline__ float pa_exp2(float x)
+{
+    float f = floorf(x);
+    if (f != f) return u2f(kQNaN);
+    uint32_t fm = f2u(f) & ~kSign;
+    if (fm == kExpo) return f > 0.0f ? f : 0.0f;
+    float t = (1.0f + x) - f;
+    float p = f >= 128.0f ? u2f(kExpo) : f <= -150.0f ? 0.0f : pow2_int((int)f);
+    return p * t;
+}
+
+// Exact derivative of a (*) b w.r.t. a, times delta (pam/native.py:65-77,
+// pam/cuda_kernels.cu:48-57): (delta * sign(b)) * 2**(e_b + [m_a + m_b >= 1]).
+__device__ __forceinline__ float pam_mul_bwd(float a, float b, float delta, float off, bool has_off)
+{
+    if (has_off) b = pam_mul(b, off);
+    uint32_t ai = f2u(a), bi = f2u(b);
+    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
+    bool fast = (mb - 0x00800000u < 0x7e800000u) & (ma - 0x00800000u < 0x7f000000u);
+    if (__builtin_expect(fast, 1))
+        return delta * u2f((bi + (ai & kMant)) & ~kMant);
+    if (mb > kExpo) return u2f(kQNaN);
+    float sgn, p;
+    if (mb == 0) { sgn = 0.0f; p = 0.0f; }
+    else if (mb == kExpo) { sgn = (bi & kSign) ? -1.0f : 1.0f; p = u2f(kExpo); }
+    else {
+        int eb; uint32_t fb; split_mag(mb, eb, fb);
+        uint32_t fa = 0;
+        if (ma != 0 && ma < kExpo) { int ea; split_mag(ma, ea, fa); }
+        sgn = (bi & kSign) ? -1.0f : 1.0f;
+        p = pow2_int(eb + (int)((fa + fb) >> 23));
+    }
+    float t = delta * sgn;
+    return t * p;
+}
+
+// Derivative of a (/) b w.r.t. b, times delta, as the reference writes it
+// (pam/cuda_kernels.cu:85-108): -(pow2 part of a (/) b) / 2^e_b * delta.
+__device__ __forceinline__ float pad_div_bwd(float a, float b, float delta, float off, bool has_off)
+{
+    float out = pad_div_off(a, b, off, has_off);
+    float om = u2f(f2u(out) & ~kMant);
+    float bm = u2f(f2u(b) & kExpo);
+    float q = om / bm;
+    return (-q) * delta;
+}
+
+// pa_exp2_bwd (pam/cuda_kernels.cu:115-123)
+__device__ __forceinline__ float pa_exp2_bwd(float x, float dy)
+{ return u2f(f2u(pa_exp2(x)) & ~kMant) * dy; }
+
+// pa_log2_bwd (pam/cuda_kernels.cu:132-136): 2**(-floor(log2 x)) * dy, x is not made positive
+__device__ __forceinline__ float pa_log2_bwd(float x, float dy)
+{
+    uint32_t xi = f2u(x), mag = xi & ~kSign;
+    if (mag > kExpo) return u2f(kQNaN);
+    float p;
+    if (mag == 0) p = u2f(kExpo);
+    else if (xi & kSign) return u2f(kQNaN);
+    else if (mag == kExpo) p = 0.0f;
+    else { int e; uint32_t m; split_mag(mag, e, m); p = pow2_int(-e); }
+    return p * dy;
+}
+
+// pa_log2 without the abs, as the reference GPU kernel has it (pam/cuda_kernels.cu:125-130)
+__device__ __forceinline__ float pa_log2_signed(float x)
+{
+    uint32_t xi = f2u(x);
+    if ((xi & kSign) && (xi & ~kSign) != 0 && (xi & ~kSign) <= kExpo) return u2f(kQNaN);
+    return pa_log2(x);
+}
+
+}  // namespace pamdev

@@ -1,0 +1,210 @@
+// Elementwise piecewise-affine kernels for gfx950: HBM-bound streams.
+//
+// One kernel template serves every op: each lane moves 128-bit vectors, a work-group
+// covers kUnroll * 256 consecutive vectors per step (so every wavefront touches whole
+// 1 KiB runs) and strides over the array by the grid size.  All loads of a step are
+// issued before the arithmetic so several are in flight per lane.
+// Algorithmic traffic: 12 B/element for the two-input forwards, 16 B/element for their
+// exact backwards, 8 B/element for pa_exp/pa_log and the scalar-operand forwards,
+// 12 B/element for the pa_exp/pa_log backwards.
+#include <math.h>
+
+#include "pam_common.h"
+#include "pam_device.h"
+
+using namespace pamdev;
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+struct OpPam {      // C = A (*) B                      (pam/cuda_kernels.cu:151)
+    float off; bool has_off;
+    __device__ float operator()(float a, float b, float) const { return pam_mul_off(a, b, off, has_off); }
+};
+struct OpPad {      // C = A (/) B                      (pam/cuda_kernels.cu:247)
+    float off; bool has_off;
+    __device__ float operator()(float a, float b, float) const { return pad_div_off(a, b, off, has_off); }
+};
+struct OpPamBwd {   // dA                               (pam/cuda_kernels.cu:196)
+    float off; bool has_off;
+    __device__ float operator()(float a, float b, float d) const { return pam_mul_bwd(a, b, d, off, has_off); }
+};
+struct OpPadBwd {   // dB                               (pam/cuda_kernels.cu:292)
+    float off; bool has_off;
+    __device__ float operator()(float a, float b, float d) const { return pad_div_bwd(a, b, d, off, has_off); }
+};
+struct OpPamBcastA { const float* s; float off; bool has_off;
+    __device__ float operator()(float x, float, float) const { return pam_mul_off(*s, x, off, has_off); } };
+struct OpPamBcastB { const float* s; float off; bool has_off;
+    __device__ float operator()(float x, float, float) const { return pam_mul_off(x, *s, off, has_off); } };
+struct OpPadBcastA { const float* s; float off; bool has_off;
+    __device__ float operator()(float x, float, float) const { return pad_div_off(*s, x, off, has_off); } };
+struct OpPadBcastB { const float* s; float off; bool has_off;
+    __device__ float operator()(float x, float, float) const { return pad_div_off(x, *s, off, has_off); } };
+struct OpExp {      // Y = pa_exp2(X (*) log2 base)     (pam/cuda_kernels.cu:344)
+    float l2b, off; bool has_off;
+    __device__ float operator()(float x, float, float) const { return pa_exp2(pam_mul_off(x, l2b, off, has_off)); }
+};
+struct OpLog {      // Y = pa_log2(X) (/) log2 base     (pam/cuda_kernels.cu:439)
+    float l2b, off; bool has_off;
+    __device__ float operator()(float x, float, float) const { return pad_div_off(pa_log2(x), l2b, off, has_off); }
+};
+struct OpExpBwd {   // (pam/cuda_kernels.cu:386-391)
+    float l2b, off; bool has_off;
+    __device__ float operator()(float x, float dy, float) const {
+        return pam_mul_bwd(x, l2b, pa_exp2_bwd(pam_mul_off(x, l2b, off, has_off), dy), off, has_off);
+    }
+};
+struct OpLogBwd {   // (pam/cuda_kernels.cu:481-484); the inner pam_bwd runs without offset
+    float l2b, off; bool has_off;
+    __device__ float operator()(float x, float dy, float) const {
+        float inv = pad_div_off(1.0f, l2b, off, has_off);
+        return pa_log2_bwd(x, pam_mul_bwd(pa_log2_signed(x), inv, dy, 1.0f, false));
+    }
+};
+
+template <class Op, int NIN>
+__global__ __launch_bounds__(kThreads) void ew_vec_kernel(const v4f* __restrict__ p0, const v4f* __restrict__ p1,
+                                                         const v4f* __restrict__ p2, v4f* __restrict__ out,
+                                                         size_t nvec, Op op)
+{
+    const size_t step = (size_t)gridDim.x * (kThreads * kUnroll);
+    for (size_t base = (size_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x; base < nvec; base += step) {
+        v4f a[kUnroll], b[kUnroll], c[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            size_t i = base + (size_t)u * kThreads;
+            if (i < nvec) {
+                a[u] = __builtin_nontemporal_load(p0 + i);
+                if (NIN > 1) b[u] = __builtin_nontemporal_load(p1 + i);
+                if (NIN > 2) c[u] = __builtin_nontemporal_load(p2 + i);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            size_t i = base + (size_t)u * kThreads;
+            if (i < nvec) {
+                v4f r;
+                r.x = op(a[u].x, NIN > 1 ? b[u].x : 0.f, NIN > 2 ? c[u].x : 0.f);
+                r.y = op(a[u].y, NIN > 1 ? b[u].y : 0.f, NIN > 2 ? c[u].y : 0.f);
+                r.z = op(a[u].z, NIN > 1 ? b[u].z : 0.f, NIN > 2 ? c[u].z : 0.f);
+                r.w = op(a[u].w, NIN > 1 ? b[u].w : 0.f, NIN > 2 ? c[u].w : 0.f);
+                __builtin_nontemporal_store(r, out + i);
+            }
+        }
+    }
+}
+
+// Unaligned pointers and the last n % 4 elements.
+template <class Op, int NIN>
+__global__ __launch_bounds__(kThreads) void ew_scalar_kernel(const float* __restrict__ p0, const float* __restrict__ p1,
+                                                            const float* __restrict__ p2, float* __restrict__ out,
+                                                            size_t first, size_t n, Op op)
+{
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (size_t i = first + (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += step)
+        out[i] = op(p0[i], NIN > 1 ? p1[i] : 0.f, NIN > 2 ? p2[i] : 0.f);
+}
+
+int g_cu_count = 0;
+
+int grid_cap()
+{
+    if (g_cu_count == 0) {
+        int dev = 0; hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256 * 8;
+        g_cu_count = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    return g_cu_count * 8;      // eight work-groups of four wavefronts per compute unit
+}
+
+template <class Op, int NIN>
+int launch(const char* what, const float* p0, const float* p1, const float* p2, float* out, size_t n, Op op, void* stream)
+{
+    if (n == 0) return PAM_HIP_OK;
+    if (!p0 || !out || (NIN > 1 && !p1) || (NIN > 2 && !p2)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: null pointer", what);
+    hipStream_t st = (hipStream_t)stream;
+    uintptr_t align = (uintptr_t)p0 | (uintptr_t)out | (NIN > 1 ? (uintptr_t)p1 : 0) | (NIN > 2 ? (uintptr_t)p2 : 0);
+    size_t nvec = (align & 15u) ? 0 : n / 4;
+    const int cap = grid_cap();
+    if (nvec) {
+        size_t blocks = (nvec + kThreads * kUnroll - 1) / (kThreads * kUnroll);
+        if (blocks > (size_t)cap) blocks = cap;
+        hipLaunchKernelGGL((ew_vec_kernel<Op, NIN>), dim3((unsigned)blocks), dim3(kThreads), 0, st,
+                           (const v4f*)p0, (const v4f*)p1, (const v4f*)p2, (v4f*)out, nvec, op);
+    }
+    if (nvec * 4 < n) {
+        size_t rest = n - nvec * 4;
+        size_t blocks = (rest + kThreads - 1) / kThreads;
+        if (blocks > (size_t)cap) blocks = cap;
+        hipLaunchKernelGGL((ew_scalar_kernel<Op, NIN>), dim3((unsigned)blocks), dim3(kThreads), 0, st,
+                           p0, p1, p2, out, nvec * 4, n, op);
+    }
+    return pamhost::check_launch(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+int pam_hip_abi_version(void) { return PAM_HIP_ABI_VERSION; }
+const char* pam_hip_last_error(void) { return pamhost::error_buffer(); }
+
+int pam_hip_device_info(int* compute_units, int* clock_khz)
+{
+    int dev = 0; hipDeviceProp_t prop;
+    hipError_t e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return pamhost::fail(PAM_HIP_ERR_LAUNCH, "device query: %s", hipGetErrorString(e));
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    return PAM_HIP_OK;
+}
+
+int pam_hip_pam_fwd(const float* a, const float* b, float* c, size_t n, float offset, void* stream)
+{ return launch<OpPam, 2>("pam_fwd", a, b, nullptr, c, n, OpPam{offset, offset != 1.0f}, stream); }
+
+int pam_hip_pad_fwd(const float* a, const float* b, float* c, size_t n, float offset, void* stream)
+{ return launch<OpPad, 2>("pad_fwd", a, b, nullptr, c, n, OpPad{offset, offset != 1.0f}, stream); }
+
+int pam_hip_pam_bwd(const float* a, const float* b, const float* dc, float* da, size_t n, float offset, void* stream)
+{ return launch<OpPamBwd, 3>("pam_bwd", a, b, dc, da, n, OpPamBwd{offset, offset != 1.0f}, stream); }
+
+int pam_hip_pad_bwd(const float* a, const float* b, const float* dc, float* db, size_t n, float offset, void* stream)
+{ return launch<OpPadBwd, 3>("pad_bwd", a, b, dc, db, n, OpPadBwd{offset, offset != 1.0f}, stream); }
+
+int pam_hip_pam_fwd_bcast(const float* x, const float* s, int scalar_is_a, float* c, size_t n, float offset, void* stream)
+{
+    if (!s) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "pam_fwd_bcast: null pointer");
+    bool ho = offset != 1.0f;
+    return scalar_is_a ? launch<OpPamBcastA, 1>("pam_fwd_bcast", x, nullptr, nullptr, c, n, OpPamBcastA{s, offset, ho}, stream)
+                       : launch<OpPamBcastB, 1>("pam_fwd_bcast", x, nullptr, nullptr, c, n, OpPamBcastB{s, offset, ho}, stream);
+}
+
+int pam_hip_pad_fwd_bcast(const float* x, const float* s, int scalar_is_a, float* c, size_t n, float offset, void* stream)
+{
+    if (!s) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "pad_fwd_bcast: null pointer");
+    bool ho = offset != 1.0f;
+    return scalar_is_a ? launch<OpPadBcastA, 1>("pad_fwd_bcast", x, nullptr, nullptr, c, n, OpPadBcastA{s, offset, ho}, stream)
+                       : launch<OpPadBcastB, 1>("pad_fwd_bcast", x, nullptr, nullptr, c, n, OpPadBcastB{s, offset, ho}, stream);
+}
+
+// log2 of the base is taken in fp32 on the host, as the reference's CPU path does with
+// torch.log2(torch.tensor(base)) (pam/native.py:203, 211-212).
+int pam_hip_pa_exp_fwd(const float* x, float* y, size_t n, float base, float offset, void* stream)
+{ return launch<OpExp, 1>("pa_exp_fwd", x, nullptr, nullptr, y, n, OpExp{log2f(base), offset, offset != 1.0f}, stream); }
+
+int pam_hip_pa_log_fwd(const float* x, float* y, size_t n, float base, float offset, void* stream)
+{ return launch<OpLog, 1>("pa_log_fwd", x, nullptr, nullptr, y, n, OpLog{log2f(base), offset, offset != 1.0f}, stream); }
+
+int pam_hip_pa_exp_bwd(const float* x, const float* dy, float* dx, size_t n, float base, float offset, void* stream)
+{ return launch<OpExpBwd, 2>("pa_exp_bwd", x, dy, nullptr, dx, n, OpExpBwd{log2f(base), offset, offset != 1.0f}, stream); }
+
+int pam_hip_pa_log_bwd(const float* x, const float* dy, float* dx, size_t n, float base, float offset, void* stream)
+{ return launch<OpLogBwd, 2>("pa_log_bwd", x, dy, nullptr, dx, n, OpLogBwd{log2f(base), offset, offset != 1.0f}, stream); }
+
+}  // extern "C"

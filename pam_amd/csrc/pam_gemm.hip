@@ -1,0 +1,556 @@
+// PAM matrix products for gfx950: Y[b,i,j] = sum_k mul(L[b,i,k], R[b,k,j]).
+//
+// A PAM product is an integer add of the two bit patterns (pam/cuda_kernels.cu:17-19),
+// so the matrix cores do not apply; this is a VALU kernel whose inner loop is, per
+// multiply-accumulate, one v_add_u32 and one v_add_f32.
+//
+//  * A work-group owns a BM x BN tile of Y.  Each lane owns a TM x TN micro-tile in
+//    registers, split into 4-wide groups spread over the tile so that the 128-bit LDS
+//    reads of a wavefront are contiguous (R fragment) or broadcast (L fragment).
+//  * L and R tiles are staged through LDS k-major ([k][row]) with a 4-word row pad, so a
+//    fragment for one k is TM/4 + TN/4 ds_read_b128.  Operands whose contiguous dimension
+//    is k (row-major L, "column-major" R) are transposed on the way in; operands whose
+//    contiguous dimension is the row are stored with 128-bit writes; anything else goes
+//    through a scalar loader.  No transposed copies are made in global memory, so the
+//    backward products run on the views the autograd layer hands over
+//    (pam/cuda_bindings.py:147-164).
+//  * Global loads for tile t+1 are issued before the arithmetic of tile t (register
+//    double buffering), LDS is double buffered, one barrier per k-tile.
+//  * The bias subtraction and the optional offset (R' = R (*) offset) are applied once per
+//    element while staging R.
+//  * While staging, every element is classified: if all of a k-tile's L and R values are
+//    normal numbers with magnitude in [2^-63, 2^64), no product in the tile can leave the
+//    normal range and the two-instruction loop is exact.  Otherwise (zeros, subnormals,
+//    inf, NaN, extreme exponents) the work-group takes a guarded loop for that k-tile,
+//    which evaluates the full definition per product.  The choice is uniform per
+//    work-group and per k-tile.
+//  * Rows beyond M / N are clamped to the last valid row when loading (their results are
+//    never stored); the k tail runs a shorter loop, padding never enters the arithmetic.
+//  * Accumulation order: every output is summed by one lane, k ascending, from +0 -- the
+//    order of the reference kernel (pam/cuda_kernels.cu:601, 608-627).  With split-K the
+//    chunk sums are added in ascending chunk order by a second kernel.
+#include "pam_common.h"
+#include "pam_device.h"
+
+using namespace pamdev;
+
+namespace {
+
+enum { MODE_PAM = 0, MODE_STD = 1, MODE_BWD_DL = 2, MODE_BWD_DR = 3 };
+enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2 };   // k contiguous / row contiguous / any strides
+
+constexpr int BK = 16;
+constexpr int PAD = 4;
+
+struct Operand { const float* p; long sb, sr, sk; };    // batch, row (the non-k index), k strides
+struct GemmArgs {
+    Operand L, R;
+    const float* D; long d_sb, d_sr, d_sc;
+    float* Y; long y_sb, y_sr, y_sc;
+    int M, N, K;
+    int ksplit, kchunk;          // kchunk is a multiple of BK; ksplit == 1 means no split
+    float off; int has_off;
+};
+
+// magnitude in [2^-63, 2^64): exponent field 64 .. 190
+__device__ __forceinline__ bool in_window(uint32_t u) { return ((u >> 23) & 0xffu) - 64u < 127u; }
+
+template <int MODE, bool IS_R>
+__device__ __forceinline__ uint32_t stage_value(float v, float off, bool has_off, bool& bad)
+{
+    // which operand carries exponent information ("b" of pam_bwd) in the backward modes
+    constexpr bool kIsSlopeSide = (MODE == MODE_BWD_DL && IS_R) || (MODE == MODE_BWD_DR && !IS_R);
+    if (MODE == MODE_STD) return f2u(v);
+    if (MODE == MODE_PAM) {
+        if (IS_R) {
+            if (has_off) v = pam_mul(v, off);
+            uint32_t u = f2u(v);
+            bad |= !in_window(u);
+            return u - kBias;
+        }
+        uint32_t u = f2u(v);
+        bad |= !in_window(u);
+        return u;
+    }
+    if (kIsSlopeSide) {
+        if (has_off) v = pam_mul(v, off);
+        uint32_t u = f2u(v);
+        bad |= !in_window(u);
+        return u;
+    }
+    uint32_t u = f2u(v);                        // the upstream gradient: zero is harmless
+    bad |= !(in_window(u) || (u & ~kSign) == 0);
+    return u;
+}
+
+// One operand's tile: ROWS x BK values from global memory into registers, then into LDS.
+template <int ROWS, int NT, int KIND>
+struct TileLoader {
+    static constexpr int kVecs = ROWS * BK / 4 / NT;      // float4 per lane (vector kinds)
+    static constexpr int kElems = ROWS * BK / NT;         // scalars per lane (generic kind)
+    static_assert(ROWS * BK % (4 * NT) == 0, "tile must divide over the work-group");
+    float4 v[kVecs > 0 ? kVecs : 1];
+
+    __device__ __forceinline__ void load(const Operand& op, const float* base, int row0, int nrows, int k0, int kend, int tid)
+    {
+        if (KIND == LOAD_KVEC) {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                int id = tid + i * NT;
+                int r = id / (BK / 4), kq = id % (BK / 4);
+                int row = min(row0 + r, nrows - 1);
+                int k = min(k0 + kq * 4, kend - 4);
+                v[i] = *reinterpret_cast<const float4*>(base + (long)row * op.sr + k);
+            }
+        } else if (KIND == LOAD_RVEC) {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                int id = tid + i * NT;
+                int k = id / (ROWS / 4), rq = id % (ROWS / 4);
+                int row = min(row0 + rq * 4, nrows - 4);
+                int kk = min(k0 + k, kend - 1);
+                v[i] = *reinterpret_cast<const float4*>(base + (long)kk * op.sk + row);
+            }
+        } else {
+            float* s = reinterpret_cast<float*>(v);
+#pragma unroll
+            for (int i = 0; i < kElems; ++i) {
+                int id = tid + i * NT;
+                int k = id / ROWS, r = id % ROWS;
+                int row = min(row0 + r, nrows - 1);
+                int kk = min(k0 + k, kend - 1);
+                s[i] = base[(long)row * op.sr + (long)kk * op.sk];
+            }
+        }
+    }
+
+    template <int MODE, bool IS_R>
+    __device__ __forceinline__ void store(uint32_t* lds, int tid, float off, bool has_off, bool& bad)
+    {
+        constexpr int LD = ROWS + PAD;
+        if (KIND == LOAD_KVEC) {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                int id = tid + i * NT;
+                int r = id / (BK / 4), kq = id % (BK / 4);
+                lds[(kq * 4 + 0) * LD + r] = stage_value<MODE, IS_R>(v[i].x, off, has_off, bad);
+                lds[(kq * 4 + 1) * LD + r] = stage_value<MODE, IS_R>(v[i].y, off, has_off, bad);
+                lds[(kq * 4 + 2) * LD + r] = stage_value<MODE, IS_R>(v[i].z, off, has_off, bad);
+                lds[(kq * 4 + 3) * LD + r] = stage_value<MODE, IS_R>(v[i].w, off, has_off, bad);
+            }
+        } else if (KIND == LOAD_RVEC) {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                int id = tid + i * NT;
+                int k = id / (ROWS / 4), rq = id % (ROWS / 4);
+                uint4 w;
+                w.x = stage_value<MODE, IS_R>(v[i].x, off, has_off, bad);
+                w.y = stage_value<MODE, IS_R>(v[i].y, off, has_off, bad);
+                w.z = stage_value<MODE, IS_R>(v[i].z, off, has_off, bad);
+                w.w = stage_value<MODE, IS_R>(v[i].w, off, has_off, bad);
+                *reinterpret_cast<uint4*>(lds + k * LD + rq * 4) = w;
+            }
+        } else {
+            const float* s = reinterpret_cast<const float*>(v);
+#pragma unroll
+            for (int i = 0; i < kElems; ++i) {
+                int id = tid + i * NT;
+                int k = id / ROWS, r = id % ROWS;
+                lds[k * LD + r] = stage_value<MODE, IS_R>(s[i], off, has_off, bad);
+            }
+        }
+    }
+};
+
+// Exact-backward product from the normalised mantissa fraction of the forward operand
+// whose gradient is wanted, the other forward operand b (offset already applied) and the
+// upstream gradient (pam/cuda_kernels.cu:48-57, pam/native.py:74-77), all classes.
+__device__ __noinline__ float bwd_product_general(uint32_t frac_a, uint32_t bi, float delta)
+{
+    uint32_t mb = bi & ~kSign;
+    if (mb > kExpo) return u2f(kQNaN);
+    float sgn, p;
+    if (mb == 0) { sgn = 0.0f; p = 0.0f; }
+    else if (mb == kExpo) { sgn = (bi & kSign) ? -1.0f : 1.0f; p = u2f(kExpo); }
+    else {
+        int eb; uint32_t fb; split_mag(mb, eb, fb);
+        sgn = (bi & kSign) ? -1.0f : 1.0f;
+        p = pow2_int(eb + (int)((frac_a + fb) >> 23));
+    }
+    float t = delta * sgn;
+    return t * p;
+}
+
+__device__ __forceinline__ uint32_t normalised_fraction(float d)
+{
+    uint32_t mag = f2u(d) & ~kSign;
+    if (mag == 0 || mag >= kExpo) return 0;       // zero; inf/NaN never carry (their fraction compares false)
+    int e; uint32_t m; split_mag(mag, e, m);
+    return m;
+}
+
+template <int BM, int BN, int TM, int TN, int MODE, int LKIND, int RKIND>
+__global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g, float* __restrict__ partial)
+{
+    constexpr int TXN = BN / TN, TYN = BM / TM, NT = TXN * TYN, NW = NT / 64;
+    constexpr int GM = TM / 4, GN = TN / 4;               // 4-wide groups per micro-tile side
+    constexpr int LDL = BM + PAD, LDR = BN + PAD;
+    static_assert(TM % 4 == 0 && TN % 4 == 0 && NT % 64 == 0, "micro-tile is built from 4-wide groups");
+
+    __shared__ __attribute__((aligned(16))) uint32_t lds_l[2][BK * LDL];
+    __shared__ __attribute__((aligned(16))) uint32_t lds_r[2][BK * LDR];
+    __shared__ uint32_t lds_flag[2][NW];
+
+    const int tid = threadIdx.x, tx = tid % TXN, ty = tid / TXN;
+    const int wave = tid / 64, lane = tid % 64;
+    const int zb = blockIdx.z / g.ksplit, zs = blockIdx.z % g.ksplit;
+    const int row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
+    const int kbegin = zs * g.kchunk;
+    const int kend = min(g.K, kbegin + g.kchunk);
+    const int ktiles = (kend - kbegin + BK - 1) / BK;
+    const bool has_off = g.has_off != 0;
+
+    const float* lbase = g.L.p + (long)zb * g.L.sb;
+    const float* rbase = g.R.p + (long)zb * g.R.sb;
+
+    float acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = 0.0f;
+
+    // forward operand whose gradient is wanted (backward modes): only its fraction matters
+    uint32_t dfrac[(MODE >= MODE_BWD_DL) ? TM : 1][(MODE >= MODE_BWD_DL) ? TN : 1];
+    if (MODE >= MODE_BWD_DL) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int r = row0 + (i / 4) * (BM / GM) + ty * 4 + (i % 4);
+                int c = col0 + (j / 4) * (BN / GN) + tx * 4 + (j % 4);
+                float d = (r < g.M && c < g.N) ? g.D[(long)zb * g.d_sb + (long)r * g.d_sr + (long)c * g.d_sc] : 0.0f;
+                dfrac[i][j] = normalised_fraction(d);
+            }
+    }
+
+    TileLoader<BM, NT, LKIND> ll;
+    TileLoader<BN, NT, RKIND> rl;
+
+    auto stage = [&](int buf) {
+        bool bad = false;
+        ll.template store<MODE, false>(lds_l[buf], tid, g.off, has_off, bad);
+        rl.template store<MODE, true>(lds_r[buf], tid, g.off, has_off, bad);
+        if (MODE != MODE_STD) {
+            unsigned long long any = __ballot(bad);
+            if (lane == 0) lds_flag[buf][wave] = any != 0ull;
+        }
+    };
+
+    if (ktiles > 0) {
+        ll.load(g.L, lbase, row0, g.M, kbegin, kend, tid);
+        rl.load(g.R, rbase, col0, g.N, kbegin, kend, tid);
+        stage(0);
+    }
+    __syncthreads();
+
+    for (int t = 0; t < ktiles; ++t) {
+        const int cur = t & 1;
+        const int k0 = kbegin + t * BK;
+        if (t + 1 < ktiles) {
+            ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid);
+            rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid);
+        }
+        const int kcount = min(BK, kend - k0);
+        bool guarded = false;
+        if (MODE != MODE_STD) {
+            uint32_t f = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) f |= lds_flag[cur][w];
+            guarded = __builtin_amdgcn_readfirstlane(f) != 0;
+        }
+        const uint32_t* sl = lds_l[cur] + ty * 4;
+        const uint32_t* sr = lds_r[cur] + tx * 4;
+
+        auto fragment = [&](int kk, uint32_t (&a)[TM], uint32_t (&b)[TN]) {
+#pragma unroll
+            for (int gi = 0; gi < GM; ++gi) {
+                uint4 q = *reinterpret_cast<const uint4*>(sl + kk * LDL + gi * (BM / GM));
+                a[gi * 4 + 0] = q.x; a[gi * 4 + 1] = q.y; a[gi * 4 + 2] = q.z; a[gi * 4 + 3] = q.w;
+            }
+#pragma unroll
+            for (int gj = 0; gj < GN; ++gj) {
+                uint4 q = *reinterpret_cast<const uint4*>(sr + kk * LDR + gj * (BN / GN));
+                b[gj * 4 + 0] = q.x; b[gj * 4 + 1] = q.y; b[gj * 4 + 2] = q.z; b[gj * 4 + 3] = q.w;
+            }
+        };
+        auto fast_step = [&](int kk) {
+            uint32_t a[TM], b[TN];
+            fragment(kk, a, b);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (MODE == MODE_PAM) acc[i][j] += u2f(a[i] + b[j]);
+                    else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(a[i]), u2f(b[j]), acc[i][j]);
+                    else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(a[i]), u2f((b[j] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                    else acc[i][j] = fmaf(u2f(b[j]), u2f((a[i] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                }
+        };
+        auto guarded_step = [&](int kk) {
+            uint32_t a[TM], b[TN];
+            fragment(kk, a, b);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if (MODE == MODE_PAM) acc[i][j] += pam_mul(u2f(a[i]), u2f(b[j] + kBias));
+                    else if (MODE == MODE_BWD_DL) acc[i][j] += bwd_product_general(dfrac[i][j], b[j], u2f(a[i]));
+                    else if (MODE == MODE_BWD_DR) acc[i][j] += bwd_product_general(dfrac[i][j], a[i], u2f(b[j]));
+                }
+        };
+
+        if (!guarded) {
+            if (kcount == BK) {
+#pragma unroll 4
+                for (int kk = 0; kk < BK; ++kk) fast_step(kk);
+            } else {
+#pragma unroll 1
+                for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
+            }
+        } else {
+#pragma unroll 1
+            for (int kk = 0; kk < kcount; ++kk) guarded_step(kk);
+        }
+
+        if (t + 1 < ktiles) stage(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: to Y, or to this chunk's slab of the split-K scratch ([chunk][batch][M][N])
+    float* out; long o_sr, o_sc;
+    if (g.ksplit > 1) {
+        out = partial + ((long)zs * (gridDim.z / g.ksplit) + zb) * (long)g.M * g.N; o_sr = g.N; o_sc = 1;
+    } else {
+        out = g.Y + (long)zb * g.y_sb; o_sr = g.y_sr; o_sc = g.y_sc;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        int r = row0 + (i / 4) * (BM / GM) + ty * 4 + (i % 4);
+        if (r >= g.M) continue;
+#pragma unroll
+        for (int gj = 0; gj < GN; ++gj) {
+            int c = col0 + gj * (BN / GN) + tx * 4;
+            float* dst = out + (long)r * o_sr + (long)c * o_sc;
+            if (o_sc == 1 && c + 3 < g.N && ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0)) {
+                *reinterpret_cast<float4*>(dst) = make_float4(acc[i][gj * 4], acc[i][gj * 4 + 1], acc[i][gj * 4 + 2], acc[i][gj * 4 + 3]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (c + j < g.N) dst[(long)j * o_sc] = acc[i][gj * 4 + j];
+            }
+        }
+    }
+}
+
+// Split-K: Y = ((0 + chunk0) + chunk1) + ... in ascending chunk order.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int chunks, long slab,
+                                                           float* __restrict__ y, long y_sb, long y_sr, long y_sc, int M, int N)
+{
+    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= slab) return;
+    float total = 0.0f;
+    for (int c = 0; c < chunks; ++c) total += partial[(long)c * slab + idx];
+    long b = idx / ((long)M * N), rem = idx % ((long)M * N);
+    y[b * y_sb + (rem / N) * y_sr + (rem % N) * y_sc] = total;
+}
+
+int g_cus = 0;
+int cu_count()
+{
+    if (g_cus == 0) {
+        int dev = 0; hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+            g_cus = prop.multiProcessorCount;
+        else
+            g_cus = 256;
+    }
+    return g_cus;
+}
+
+struct Plan { int big; int ksplit; int kchunk; };
+
+// Tile shape and split-K factor for a problem.  128x128 tiles (8x8 per lane) when they
+// fill the device, 64x64 (4x4 per lane) otherwise; K is split when even the small tiles
+// leave most compute units idle and K is long.
+Plan make_plan(long batch, long M, long N, long K, bool allow_split)
+{
+    const long cus = cu_count();
+    auto tiles = [&](long bm, long bn) { return batch * ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    Plan p{0, 1, (int)((K + BK - 1) / BK * BK)};
+    if (p.kchunk == 0) p.kchunk = BK;
+    if (tiles(128, 128) >= 2 * cus) { p.big = 1; return p; }
+    long t = tiles(64, 64);
+    long ktiles = (K + BK - 1) / BK;
+    if (allow_split && t < 2 * cus && ktiles >= 16) {
+        long want = (4 * cus + t - 1) / t;                  // aim at ~4 work-groups per compute unit
+        long maxsplit = ktiles / 8;                        // at least 8 k-tiles (128 k) per chunk
+        long s = want < maxsplit ? want : maxsplit;
+        if (s > 1) {
+            long per = (ktiles + s - 1) / s;
+            p.kchunk = (int)(per * BK);
+            p.ksplit = (int)((ktiles + per - 1) / per);
+        }
+    }
+    return p;
+}
+
+int load_kind(long s_row, long s_k, long s_batch, const float* p, long rows, long K)
+{
+    bool aligned = ((reinterpret_cast<uintptr_t>(p) & 15u) == 0) && (s_batch % 4 == 0);
+    if (s_k == 1 && aligned && s_row % 4 == 0 && K % 4 == 0 && K >= 4) return LOAD_KVEC;
+    if (s_row == 1 && aligned && s_k % 4 == 0 && rows % 4 == 0 && rows >= 4) return LOAD_RVEC;
+    return LOAD_ANY;
+}
+
+template <int BM, int BN, int TM, int TN, int MODE>
+void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, float* partial)
+{
+    constexpr int NT = (BM / TM) * (BN / TN);
+#define PAM_GEMM_CASE(LK, RK) \
+    if (lk == LK && rk == RK) { hipLaunchKernelGGL((gemm_kernel<BM, BN, TM, TN, MODE, LK, RK>), grid, dim3(NT), 0, st, g, partial); return; }
+    PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
+    PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
+    PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
+#undef PAM_GEMM_CASE
+}
+
+template <int MODE>
+void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& g, long batch, float* partial)
+{
+    if (p.big) {
+        dim3 grid((g.N + 127) / 128, (g.M + 127) / 128, (unsigned)(batch * p.ksplit));
+        launch_kinds<128, 128, 8, 8, MODE>(lk, rk, grid, st, g, partial);
+    } else {
+        dim3 grid((g.N + 63) / 64, (g.M + 63) / 64, (unsigned)(batch * p.ksplit));
+        launch_kinds<64, 64, 4, 4, MODE>(lk, rk, grid, st, g, partial);
+    }
+}
+
+int gemm(const char* what, int mode, long batch, long M, long N, long K,
+         const float* l, long l_sb, long l_sr, long l_sc, const float* r, long r_sb, long r_sr, long r_sc,
+         const float* d, long d_sb, long d_sr, long d_sc, float* y, long y_sb, long y_sr, long y_sc,
+         float offset, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (batch < 0 || M < 0 || N < 0 || K < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: negative size", what);
+    if (batch == 0 || M == 0 || N == 0) return PAM_HIP_OK;
+    if (!l || !r || !y || (mode >= MODE_BWD_DL && !d)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: null pointer", what);
+    if (M > 0x7ffffff0L || N > 0x7ffffff0L || K > 0x7ffffff0L)
+        return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: dimension beyond 2^31", what);
+    hipStream_t st = (hipStream_t)stream;
+
+    Plan p = make_plan(batch, M, N, K, workspace != nullptr);
+    if (batch * p.ksplit > 65535) { p.ksplit = 1; p.kchunk = (int)((K + BK - 1) / BK * BK); }
+    if (batch > 65535) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: batch beyond 65535", what);
+    if (p.ksplit > 1) {
+        size_t need = (size_t)p.ksplit * batch * M * N * sizeof(float);
+        if (need > workspace_bytes) { p.ksplit = 1; p.kchunk = (int)((K + BK - 1) / BK * BK); }
+    }
+    if (p.kchunk < BK) p.kchunk = BK;
+
+    GemmArgs g;
+    g.L = Operand{l, l_sb, l_sr, l_sc};
+    g.R = Operand{r, r_sb, r_sc, r_sr};            // R's "row" index is the output column
+    g.D = d; g.d_sb = d_sb; g.d_sr = d_sr; g.d_sc = d_sc;
+    g.Y = y; g.y_sb = y_sb; g.y_sr = y_sr; g.y_sc = y_sc;
+    g.M = (int)M; g.N = (int)N; g.K = (int)K;
+    g.ksplit = p.ksplit; g.kchunk = p.kchunk;
+    g.off = offset; g.has_off = (mode != MODE_STD && offset != 1.0f) ? 1 : 0;
+
+    int lk = load_kind(l_sr, l_sc, l_sb, l, M, K);
+    int rk = load_kind(r_sc, r_sr, r_sb, r, N, K);
+    float* partial = (float*)workspace;
+    switch (mode) {
+    case MODE_PAM: launch_mode<MODE_PAM>(p, lk, rk, st, g, batch, partial); break;
+    case MODE_STD: launch_mode<MODE_STD>(p, lk, rk, st, g, batch, partial); break;
+    case MODE_BWD_DL: launch_mode<MODE_BWD_DL>(p, lk, rk, st, g, batch, partial); break;
+    default: launch_mode<MODE_BWD_DR>(p, lk, rk, st, g, batch, partial); break;
+    }
+    if (p.ksplit > 1) {
+        long slab = batch * M * N;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((slab + 255) / 256)), dim3(256), 0, st,
+                           partial, p.ksplit, slab, y, y_sb, y_sr, y_sc, (int)M, (int)N);
+    }
+    return pamhost::check_launch(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t pam_hip_gemm_workspace_bytes(long batch, long m, long n, long k)
+{
+    if (batch <= 0 || m <= 0 || n <= 0 || k <= 0) return 0;
+    Plan p = make_plan(batch, m, n, k, true);
+    return p.ksplit > 1 ? (size_t)p.ksplit * batch * m * n * sizeof(float) : 0;
+}
+
+int pam_hip_gemm_plan(long batch, long m, long n, long k, int* k_splits, int* k_chunk)
+{
+    if (batch <= 0 || m <= 0 || n <= 0 || k < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "gemm_plan: bad shape");
+    Plan p = make_plan(batch, m, n, k, true);
+    if (batch * p.ksplit > 65535) { p.ksplit = 1; p.kchunk = (int)((k + BK - 1) / BK * BK); }
+    if (k_splits) *k_splits = p.ksplit;
+    if (k_chunk) *k_chunk = p.ksplit > 1 ? p.kchunk : (int)k;
+    return PAM_HIP_OK;
+}
+
+int pam_hip_pam_matmul_fwd(const float* a, long a_sr, long a_sc, const float* b, long b_sr, long b_sc,
+                           float* y, long y_sr, long y_sc, long m, long n, long k, float offset,
+                           void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm("pam_matmul_fwd", MODE_PAM, 1, m, n, k, a, 0, a_sr, a_sc, b, 0, b_sr, b_sc, nullptr, 0, 0, 0,
+                y, 0, y_sr, y_sc, offset, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_pam_bmm_fwd(PAM_HIP_MAT(a), PAM_HIP_MAT(b), PAM_HIP_OUT(y), long batch, long m, long n, long k,
+                        float offset, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm("pam_bmm_fwd", MODE_PAM, batch, m, n, k, a, a_sb, a_sr, a_sc, b, b_sb, b_sr, b_sc, nullptr, 0, 0, 0,
+                y, y_sb, y_sr, y_sc, offset, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_standard_matmul(const float* a, long a_sr, long a_sc, const float* b, long b_sr, long b_sc,
+                            float* y, long y_sr, long y_sc, long m, long n, long k, float ignored,
+                            void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)ignored;
+    return gemm("standard_matmul", MODE_STD, 1, m, n, k, a, 0, a_sr, a_sc, b, 0, b_sr, b_sc, nullptr, 0, 0, 0,
+                y, 0, y_sr, y_sc, 1.0f, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_standard_bmm(PAM_HIP_MAT(a), PAM_HIP_MAT(b), PAM_HIP_OUT(y), long batch, long m, long n, long k,
+                         float ignored, void* workspace, size_t workspace_bytes, void* stream)
+{
+    (void)ignored;
+    return gemm("standard_bmm", MODE_STD, batch, m, n, k, a, a_sb, a_sr, a_sc, b, b_sb, b_sr, b_sc, nullptr, 0, 0, 0,
+                y, y_sb, y_sr, y_sc, 1.0f, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_pam_matmul_bwd(const float* l, long l_sr, long l_sc, const float* r, long r_sr, long r_sc,
+                           const float* mo, long mo_sr, long mo_sc, float* dm, long dm_sr, long dm_sc,
+                           long m, long n, long k, int delta_l, float offset,
+                           void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm("pam_matmul_bwd", delta_l ? MODE_BWD_DL : MODE_BWD_DR, 1, m, n, k, l, 0, l_sr, l_sc, r, 0, r_sr, r_sc,
+                mo, 0, mo_sr, mo_sc, dm, 0, dm_sr, dm_sc, offset, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_pam_bmm_bwd(PAM_HIP_MAT(l), PAM_HIP_MAT(r), PAM_HIP_MAT(mo), PAM_HIP_OUT(dm),
+                        long batch, long m, long n, long k, int delta_l, float offset,
+                        void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm("pam_bmm_bwd", delta_l ? MODE_BWD_DL : MODE_BWD_DR, batch, m, n, k, l, l_sb, l_sr, l_sc, r, r_sb, r_sr, r_sc,
+                mo, mo_sb, mo_sr, mo_sc, dm, dm_sb, dm_sr, dm_sc, offset, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,375 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C ABI, on a real MI355X.
+
+Bars: bit-exact (NaN compared as a class) against the oracle's exact flavour for every
+elementwise op and for matrix products in the fixed accumulation order; against the
+golden vectors written from the reference's pam/native.py: bit-exact where its float
+emulation is exact, and its own allclose(rtol=1e-5, atol=1e-8) elsewhere, with every
+differing element required to be one the oracle's model of that emulation reproduces.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from _util import GOLDEN, assert_same_bits, below_pow2, edge_values, f32, fclass, mixed_operands, same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from pam_amd._abi import HipKernels, load_library
+    load_library()
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return HipKernels()
+
+
+def dev(x):
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.detach().cpu().numpy()
+
+
+OFFS = [None, 1.0552]
+
+
+def _o(off):
+    return 1.0 if off is None else off
+
+
+# ------------------------------------------------------------------ elementwise vs oracle
+
+@pytest.mark.parametrize("off", OFFS)
+def test_pam_pad_mixed(K, oracle, off):
+    n = (1 << 20) + 3
+    a, b = mixed_operands(n, 10), mixed_operands(n, 11)
+    assert_same_bits(host(K.pam_fwd(dev(a), dev(b), _o(off))), oracle.pam(a, b, off), "pam_fwd")
+    assert_same_bits(host(K.pad_fwd(dev(a), dev(b), _o(off))), oracle.pad(a, b, off), "pad_fwd")
+
+
+@pytest.mark.parametrize("off", OFFS)
+def test_edge_grid_all_pairs(K, oracle, off):
+    ev = edge_values()
+    a = np.repeat(ev, len(ev)); b = np.tile(ev, len(ev))
+    assert_same_bits(host(K.pam_fwd(dev(a), dev(b), _o(off))), oracle.pam(a, b, off), "pam_fwd")
+    assert_same_bits(host(K.pad_fwd(dev(a), dev(b), _o(off))), oracle.pad(a, b, off), "pad_fwd")
+    d = np.resize(np.array([1.0, -3.0, 0.0, np.inf, 1e-40, np.nan, 2.5e38], np.float32), a.size)
+    assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), _o(off))), oracle.pam_bwd(a, b, d, off), "pam_bwd")
+    assert_same_bits(host(K.pad_bwd(dev(a), dev(b), dev(d), _o(off))), oracle.pad_bwd(a, b, d, off), "pad_bwd")
+
+
+@pytest.mark.parametrize("off", OFFS)
+def test_exact_backward_mixed(K, oracle, off):
+    n = (1 << 18) + 1
+    a, b, d = mixed_operands(n, 20), mixed_operands(n, 21), mixed_operands(n, 22, edge_frac=0.005)
+    assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), _o(off))), oracle.pam_bwd(a, b, d, off), "pam_bwd")
+    assert_same_bits(host(K.pad_bwd(dev(a), dev(b), dev(d), _o(off))), oracle.pad_bwd(a, b, d, off), "pad_bwd")
+
+
+@pytest.mark.parametrize("off", OFFS)
+@pytest.mark.parametrize("base", [math.e, 2.0, 10.0, 0.5])
+def test_exp_log(K, oracle, base, off):
+    rng = np.random.RandomState(30)
+    xs = np.concatenate([np.linspace(-160, 160, 4097), rng.standard_normal(1 << 16) * 8, edge_values(),
+                         [127.5, 128.0, -149.0, -149.5, -150.0, 2.0 ** 24, 2.0 ** 25, 1e30, -1e30]]).astype(np.float32)
+    xl = np.concatenate([rng.rand(1 << 16) * 10, 2.0 ** (rng.rand(1 << 14) * 250 - 125), edge_values()]).astype(np.float32)
+    dy = np.resize(mixed_operands(4099, 31, edge_frac=0.01), xs.size)
+    assert_same_bits(host(K.pa_exp_fwd(dev(xs), base, _o(off))), oracle.pa_exp(xs, base, off), "pa_exp_fwd")
+    assert_same_bits(host(K.pa_log_fwd(dev(xl), base, _o(off))), oracle.pa_log(xl, base, off), "pa_log_fwd")
+    assert_same_bits(host(K.pa_exp_bwd(dev(xs), dev(dy), base, _o(off))), oracle.pa_exp_bwd(xs, dy, base, off), "pa_exp_bwd")
+    dyl = np.resize(dy, xl.size)
+    assert_same_bits(host(K.pa_log_bwd(dev(xl), dev(dyl), base, _o(off))), oracle.pa_log_bwd(xl, dyl, base, off), "pa_log_bwd")
+
+
+def test_ragged_unaligned_and_broadcast(K, oracle):
+    for n in (0, 1, 3, 5, 1023, 1025, 4099):
+        a, b = mixed_operands(n + 1, 40 + n), mixed_operands(n + 1, 41 + n)
+        # views that start 4 bytes into an allocation: the vector path must not be taken
+        ta, tb = dev(a)[1:], dev(b)[1:]
+        assert_same_bits(host(K.pam_fwd(ta, tb, 1.0)), oracle.pam(a[1:], b[1:]), f"pam n={n}")
+        assert_same_bits(host(K.pad_fwd(ta, dev(b[1:]), 1.0)), oracle.pad(a[1:], b[1:]), f"pad n={n}")
+    a = mixed_operands(70001, 50)
+    for s in (1.5, 0.0, -0.0, float("inf"), 1e-41, -3.0e38):
+        st = torch.tensor(s, device="cuda")
+        A = dev(a[:70000]).reshape(7, 10000)
+        assert_same_bits(host(K.pam_fwd(A, st.expand(A.shape), 1.0552)), oracle.pam(a[:70000].reshape(7, 10000), np.float32(s), 1.0552), "pam x*s")
+        assert_same_bits(host(K.pam_fwd(st.expand(A.shape), A, 1.0)), oracle.pam(np.float32(s), a[:70000].reshape(7, 10000)), "pam s*x")
+        assert_same_bits(host(K.pad_fwd(A, st.expand(A.shape), 1.0)), oracle.pad(a[:70000].reshape(7, 10000), np.float32(s)), "pad x/s")
+        assert_same_bits(host(K.pad_fwd(st.expand(A.shape), A, 1.0552)), oracle.pad(np.float32(s), a[:70000].reshape(7, 10000), 1.0552), "pad s/x")
+    # non-contiguous input (transposed view): copied like the reference's flatten()
+    m = mixed_operands(6 * 50, 51).reshape(6, 50)
+    assert_same_bits(host(K.pam_fwd(dev(m).T, dev(m.T.copy()), 1.0)), oracle.pam(m.T, m.T), "transposed view")
+
+
+# ------------------------------------------------------------------ elementwise vs native.py goldens
+
+def test_goldens_short_mantissa_bit_exact(K):
+    g = np.load(GOLDEN / "short_mantissa.npz")
+    a, b, d = f32(g["a"]), f32(g["b"]), f32(g["d"])
+    assert_same_bits(host(K.pam_fwd(dev(a), dev(b), 1.0)), f32(g["pam"]), "pam vs native.py")
+    assert_same_bits(host(K.pad_fwd(dev(a), dev(b), 1.0)), f32(g["pad"]), "pad vs native.py")
+    assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), 1.0)), f32(g["pam_bwd"]), "pam_bwd vs native.py")
+
+
+def test_goldens_full_mantissa(K, oracle):
+    g = np.load(GOLDEN / "normal_fullmant.npz")
+    a, b, d = f32(g["a"]), f32(g["b"]), f32(g["d"]); off = float(g["offset"])
+    cases = [("pam", K.pam_fwd, oracle.pam_chain, None), ("pad", K.pad_fwd, oracle.pad_chain, None),
+             ("pam_off", K.pam_fwd, oracle.pam_chain, off), ("pad_off", K.pad_fwd, oracle.pad_chain, off)]
+    for name, fn, chain, o in cases:
+        got = host(fn(dev(a), dev(b), _o(o))); want = f32(g[name])
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-8), name           # the reference's own bar
+        differ = ~same_bits(got, want)
+        # every element where the integer add and native.py disagree is one where the model of
+        # native.py's float chain reproduces native.py: the difference is its rounding, not ours
+        assert same_bits(chain(a, b, o), want)[differ].all(), name
+    assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), 1.0)), f32(g["pam_bwd"]), "pam_bwd")
+    assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), off)), f32(g["pam_bwd_off"]), "pam_bwd offset")
+
+
+def test_goldens_edge_grid_classes(K):
+    g = np.load(GOLDEN / "edge_grid.npz")
+    ev = f32(g["values"]); a = np.repeat(ev, len(ev)); b = np.tile(ev, len(ev))
+    keep = ~(below_pow2(a) | below_pow2(b))
+    for name, fn, o in (("pam", K.pam_fwd, 1.0), ("pad", K.pad_fwd, 1.0),
+                        ("pam_off", K.pam_fwd, float(g["offset"])), ("pad_off", K.pad_fwd, float(g["offset"]))):
+        got = host(fn(dev(a), dev(b), o))[keep]; want = f32(g[name])[keep]
+        assert (fclass(got) == fclass(want)).all(), name
+        nn = ~np.isnan(want)
+        assert (np.signbit(got[nn]) == np.signbit(want[nn])).all(), name        # signed zeros and infinities
+        fin = fclass(want) == 1
+        rel = np.abs(got[fin].astype(np.float64) - want[fin]) / np.abs(want[fin].astype(np.float64))
+        assert rel.max() <= 2.0 ** -16, name
+
+
+def test_goldens_exp_log(K, oracle):
+    g = np.load(GOLDEN / "exp_log.npz")
+    xs, xl = f32(g["x_exp"]), f32(g["x_log"])
+    ok_s, ok_l = ~below_pow2(xs), ~below_pow2(xl)
+    for name, base in (("e", math.e), ("2", 2.0), ("10", 10.0)):
+        got = host(K.pa_exp_fwd(dev(xs), base, 1.0))[ok_s]; want = f32(g[f"exp_{name}"])[ok_s]
+        differ = ~same_bits(got, want)
+        assert same_bits(oracle.pa_exp_chain(xs, base)[ok_s], want)[differ].all()
+        sel = (fclass(want) == 1) & (np.abs(want) > 1e-30)
+        assert np.allclose(got[sel], want[sel], rtol=3e-4, atol=1e-6)
+        got = host(K.pa_log_fwd(dev(xl), base, 1.0))[ok_l]; want = f32(g[f"log_{name}"])[ok_l]
+        differ = ~same_bits(got, want)
+        assert same_bits(oracle.pa_log_chain(xl, base)[ok_l], want)[differ].all()
+        sel = fclass(want) == 1
+        assert np.allclose(got[sel], want[sel], rtol=3e-4, atol=1e-6)
+
+
+# ------------------------------------------------------------------ matrix products vs oracle
+
+def _layouts(x):
+    """row-major, column-major (transposed storage) and a generic-stride view of the same matrix"""
+    t = dev(x)
+    cm = dev(np.ascontiguousarray(np.swapaxes(x, -1, -2))).transpose(-1, -2)
+    wide = torch.zeros(*x.shape[:-1], x.shape[-1] * 2 + 1, device="cuda")
+    wide[..., ::2][..., :x.shape[-1]] = t
+    return {"rm": t, "cm": cm, "any": wide[..., ::2][..., :x.shape[-1]]}
+
+
+def _rand(shape, seed, zeros=0.0, specials=False):
+    rng = np.random.RandomState(seed)
+    x = rng.standard_normal(shape).astype(np.float32)
+    if zeros:
+        x[rng.rand(*shape) < zeros] = 0.0
+    if specials:
+        flat = x.reshape(-1)
+        idx = rng.choice(flat.size, size=max(4, flat.size // 200), replace=False)
+        flat[idx] = np.resize(np.array([np.inf, -0.0, 1e-40, np.nan, 3e38, -1e-39, 2.0 ** -100, 2.0 ** 100], np.float32), idx.size)
+    return x
+
+
+SHAPES = [(5, 4, 3), (64, 16, 64), (70, 33, 45), (130, 100, 257), (128, 197, 128), (33, 1, 9), (257, 64, 192)]
+
+
+@pytest.mark.parametrize("m,k,n", SHAPES)
+def test_matmul_forward_layouts(K, oracle, m, k, n):
+    A, B = _rand((m, k), m + k), _rand((k, n), n + k + 1)
+    want = oracle.gemm(A, B)
+    for la, ta in _layouts(A).items():
+        for lb, tb in _layouts(B).items():
+            assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), want, f"{la} x {lb}")
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), oracle.gemm(A, B, offset=1.0552), "offset")
+    assert_same_bits(host(K.standard_matmul(dev(A), dev(B), True, True, 1.0)), oracle.gemm(A, B, mode=oracle.MODE_STD), "standard")
+
+
+@pytest.mark.parametrize("zeros,specials", [(0.5, False), (0.02, True), (1.0, False)])
+def test_matmul_zeros_and_specials(K, oracle, zeros, specials):
+    A, B = _rand((150, 75), 1, zeros, specials), _rand((75, 90), 2, zeros / 2, specials)
+    for la, ta in _layouts(A).items():
+        for lb, tb in _layouts(B).items():
+            assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), oracle.gemm(A, B), f"{la} x {lb}")
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), oracle.gemm(A, B, offset=1.0552), "offset")
+
+
+@pytest.mark.parametrize("delta_l", [True, False])
+@pytest.mark.parametrize("zeros,specials", [(0.0, False), (0.3, True)])
+def test_matmul_exact_backward(K, oracle, delta_l, zeros, specials):
+    L, R, D = _rand((70, 45), 3, zeros, specials), _rand((45, 97), 4, zeros, specials), _rand((70, 97), 5, zeros / 3, specials)
+    mode = oracle.MODE_BWD_DELTA_L if delta_l else oracle.MODE_BWD_DELTA_R
+    for off in OFFS:
+        want = oracle.gemm(L, R, mode=mode, D=D, offset=off)
+        for ll, tl in _layouts(L).items():
+            for lr, tr in _layouts(R).items():
+                got = host(K.pam_matmul_bwd(tl, tr, dev(D), True, True, delta_l, _o(off)))
+                assert_same_bits(got, want, f"{ll} x {lr} off={off}")
+
+
+def test_bmm_tails_and_strides(K, oracle):
+    # the reference's own bmm test shape (pam/test_pam.py:198-205): power-of-two weights => equals bmm
+    rng = np.random.RandomState(6)
+    X = (rng.randint(-128, 128, (11, 13, 15)) / 64.0).astype(np.float32)
+    W = (2.0 ** rng.randint(-8, 8, (11, 15, 19))).astype(np.float32)
+    got = host(K.pam_bmm_fwd(dev(X), dev(W), True, True, 1.0))
+    assert_same_bits(got, np.matmul(X.astype(np.float64), W.astype(np.float64)).astype(np.float32), "pow2 bmm")
+    # attention-shaped operands, K = 197 (prime) and 64, every layout
+    Q, Kt = _rand((6, 197, 64), 7), _rand((6, 64, 197), 8)
+    P, V = _rand((6, 197, 197), 9, zeros=0.1), _rand((6, 197, 64), 10)
+    for L, R in ((Q, Kt), (P, V)):
+        want = oracle.gemm(L, R)
+        for ll, tl in _layouts(L).items():
+            for lr, tr in _layouts(R).items():
+                assert_same_bits(host(K.pam_bmm_fwd(tl, tr, True, True, 1.0)), want, f"bmm {ll} x {lr}")
+    D = _rand((6, 197, 64), 11)
+    assert_same_bits(host(K.pam_bmm_bwd(dev(P), dev(V), dev(D), True, True, True, 1.0)),
+                     oracle.gemm(P, V, mode=oracle.MODE_BWD_DELTA_L, D=D), "bmm bwd")
+    # fairseq-style strided batch: q = x.view(T, B*H, D).transpose(0, 1), batch stride < row stride
+    T, BH, Dh = 32, 12, 16
+    x = _rand((T, BH, Dh), 12); y = _rand((T, BH, Dh), 13)
+    q = dev(x).transpose(0, 1); kt = dev(y).transpose(0, 1).transpose(1, 2)
+    assert q.stride() == (Dh, BH * Dh, 1) and kt.stride() == (Dh, 1, BH * Dh)
+    want = oracle.gemm(np.swapaxes(x, 0, 1), np.swapaxes(np.swapaxes(y, 0, 1), 1, 2))
+    assert_same_bits(host(K.pam_bmm_fwd(q, kt, True, False, 1.0)), want, "strided batch")
+
+
+def test_split_k_fixed_order(K, oracle):
+    from pam_amd import _abi
+    m, n, k = 96, 160, 4096
+    splits, chunk = _abi.gemm_plan(1, m, n, k)
+    assert splits > 1 and chunk % 16 == 0
+    A, B = _rand((m, k), 14), _rand((k, n), 15)
+    want = oracle.gemm(A, B, kchunk=chunk)
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)), want, "split-K order")
+    At = dev(np.ascontiguousarray(A.T)).T                      # the dW layout: column-major left operand
+    assert_same_bits(host(K.pam_matmul_fwd(At, dev(B), False, True, 1.0)), want, "split-K, cm x rm")
+
+
+def test_matmul_config0_golden(K, oracle):
+    from test_oracle_goldens import c0_operands
+    g = np.load(GOLDEN / "matmul_c0.npz")
+    A, B, dY = c0_operands()
+    Y = host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)); want = f32(g["y"]).reshape(256, 256)
+    assert_same_bits(Y, oracle.gemm(A, B, kchunk=_plan_chunk(256, 256, 512)), "config 0 forward vs oracle")
+    assert np.abs(Y - want).max() / np.abs(want).max() <= 1e-5                  # vs native.pam_matmul
+    dA = host(K.pam_matmul_fwd(dev(dY), dev(B).T, True, False, 1.0))
+    dB = host(K.pam_matmul_fwd(dev(A).T, dev(dY), False, True, 1.0))
+    assert np.abs(dA[::8] - f32(g["da_rows"]).reshape(32, 512)).max() / np.abs(f32(g["da_rows"])).max() <= 1e-5
+    assert np.abs(dB[::8] - f32(g["db_rows"]).reshape(64, 256)).max() / np.abs(f32(g["db_rows"])).max() <= 1e-5
+
+
+def _plan_chunk(m, n, k, batch=1):
+    from pam_amd import _abi
+    splits, chunk = _abi.gemm_plan(batch, m, n, k)
+    return chunk if splits > 1 else 0
+
+
+# ------------------------------------------------------------------ full-size configurations
+
+def test_deit_linear_full_size(K, oracle):
+    """12608 x 192 -> 768 forward and both backward products at full size: sampled rows
+    against the oracle, and exact scale-invariance of the whole result."""
+    rng = np.random.RandomState(100)
+    X = rng.standard_normal((12608, 192)).astype(np.float32)
+    W = np.clip(rng.standard_normal((768, 192)) * 0.02, -0.04, 0.04).astype(np.float32)
+    dY = (rng.standard_normal((12608, 768)) * 1e-2).astype(np.float32)
+    tX, tW, tdY = dev(X), dev(W), dev(dY)
+    Y = K.pam_matmul_fwd(tX, tW.T, True, False, 1.0)
+    dX = K.pam_matmul_fwd(tdY, tW, True, True, 1.0)
+    dW = K.pam_matmul_fwd(tX.T, tdY, False, True, 1.0)
+    rows = rng.choice(12608, 48, replace=False)
+    assert_same_bits(host(Y)[rows], oracle.gemm(X[rows], W.T, kchunk=_plan_chunk(12608, 768, 192)), "Y rows")
+    assert_same_bits(host(dX)[rows], oracle.gemm(dY[rows], W, kchunk=_plan_chunk(12608, 192, 768)), "dX rows")
+    cols = rng.choice(768, 24, replace=False)
+    assert_same_bits(host(dW)[:, cols], oracle.gemm(X.T, dY[:, cols], kchunk=_plan_chunk(192, 768, 12608)), "dW cols")
+    # multiplying an operand by a power of two multiplies every PAM product, hence the sum, exactly
+    assert torch.equal(K.pam_matmul_fwd(tX * 4.0, tW.T, True, False, 1.0), Y * 4.0)
+    assert torch.equal(K.pam_matmul_fwd(tX, (tW * 0.5).T, True, False, 1.0), Y * 0.5)
+    # a row permutation of X permutes the rows of Y
+    perm = torch.randperm(12608, device="cuda")
+    assert torch.equal(K.pam_matmul_fwd(tX[perm], tW.T, True, False, 1.0), Y[perm])
+
+
+def test_elementwise_full_size(K, oracle):
+    """2^26 elements, 98 % N(0,1) and 2 % edge values: slices against the oracle, and the
+    round trip (a (*) b) (/) b == a wherever nothing saturates."""
+    n = 1 << 26
+    a, b = mixed_operands(n, 10), mixed_operands(n, 11)
+    ta, tb = dev(a), dev(b)
+    prod = K.pam_fwd(ta, tb, 1.0); quot = K.pad_fwd(ta, tb, 1.0)
+    hp, hq = host(prod), host(quot)
+    for lo in (0, 12345677, n - (1 << 20)):
+        sl = slice(lo, lo + (1 << 20))
+        assert_same_bits(hp[sl], oracle.pam(a[sl], b[sl]), f"pam slice {lo}")
+        assert_same_bits(hq[sl], oracle.pad(a[sl], b[sl]), f"pad slice {lo}")
+    back = host(K.pad_fwd(prod, tb, 1.0))
+    ea = (a.view(np.uint32) >> 23) & 0xff; eb = (b.view(np.uint32) >> 23) & 0xff
+    safe = (ea > 40) & (ea < 210) & (eb > 40) & (eb < 210)
+    assert safe.mean() > 0.95 and (back[safe].view(np.uint32) == a[safe].view(np.uint32)).all()
+    # checksum of the whole array against the oracle on all host cores
+    want = oracle.pam(a, b)
+    assert np.bitwise_xor.reduce(hp.view(np.uint32)[~np.isnan(hp)]) == np.bitwise_xor.reduce(want.view(np.uint32)[~np.isnan(want)])
+    assert (np.isnan(hp) == np.isnan(want)).all()
+
+
+# ------------------------------------------------------------------ autograd layer on the device
+
+def test_linear_autograd_matches_oracle(K, oracle):
+    import pam_amd as pam
+    rng = np.random.RandomState(200)
+    X = rng.standard_normal((4, 50, 96)).astype(np.float32); W = (rng.standard_normal((40, 96)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(40).astype(np.float32); dY = rng.standard_normal((4, 50, 40)).astype(np.float32)
+    for approx in (True, False):
+        lin = pam.Linear(96, 40, approx_bwd=approx).cuda()
+        with torch.no_grad():
+            lin.weight.copy_(dev(W)); lin.bias.copy_(dev(bias))
+        x = dev(X).requires_grad_()
+        y = lin(x); y.backward(dev(dY))
+        X2, dY2 = X.reshape(200, 96), dY.reshape(200, 40)
+        assert_same_bits(host(y).reshape(200, 40), oracle.gemm(X2, W.T) + bias, "linear forward")
+        if approx:
+            assert_same_bits(host(x.grad).reshape(200, 96), oracle.gemm(dY2, W), "dX approx")
+            assert_same_bits(host(lin.weight.grad), oracle.gemm(X2.T, dY2).T, "dW approx")
+        else:
+            assert_same_bits(host(x.grad).reshape(200, 96), oracle.gemm(dY2, W, mode=oracle.MODE_BWD_DELTA_L, D=X2), "dX exact")
+            assert_same_bits(host(lin.weight.grad), oracle.gemm(X2.T, dY2, mode=oracle.MODE_BWD_DELTA_R, D=W.T).T, "dW exact")
+
+
+def test_reference_vectors_on_device(K):
+    # pam/test_pam.py:13-45 run against the HIP path, with the reference's comparators
+    import pam_amd as pam
+    abc = torch.tensor([
+        [1.0, 1.0, 1.0], [1.2345, 1.0, 1.2345], [1.2345, 32.0, 32.0 * 1.2345], [-1.2345, 32.0, -32.0 * 1.2345],
+        [1.2345, -32.0, -32.0 * 1.2345], [-1.2345, -32.0, 32.0 * 1.2345], [1.0, 0.0, 0.0], [0.0, -1.0, -0.0],
+        [1.5, 1.5, 2.0], [1.3, -1.3, -1.6], [4.5, 3.0, 8 * (1 + (4.5 - 4) / 4 + (3.0 - 2) / 2)], [-6.0, 3.0, -16.0],
+        [-3.5, -3.5, 8 * (1 + (3.5 - 2) / 2 + (3.5 - 2) / 2 - 1)], [1e-30, 1e-30, 0.0], [1e-30, -1e-30, -0.0]], device="cuda")
+    assert torch.allclose(abc[:, 2], pam.mul(abc[:, 0].contiguous(), abc[:, 1].contiguous()))
+    ab = torch.tensor([[1e30, 1e30], [1e30, -1e30], [float("-inf"), 1e-20], [float("nan"), -1e-20],
+                       [float("inf"), 0.0], [float("nan"), 0.0]], device="cuda")
+    assert (~pam.mul(ab[:, 0].contiguous(), ab[:, 1].contiguous()).isfinite()).all()
+    # pam/test_pam.py:127-148: approximate backward equals the two transposed products
+    A = (torch.arange(20) ** 3 % 7 - 2.0).reshape((5, 4)).cuda().requires_grad_()
+    B = (torch.arange(12) ** 2 % 5 - 2.0).reshape((3, 4)).T.cuda().requires_grad_()
+    C = pam.matmul(A, B, approx_bwd=True)
+    delta = torch.arange(C.numel()).float().reshape_as(C).cuda()
+    C.backward(delta)
+    assert torch.equal(A.grad, pam.matmul(delta, B.detach().T)) and torch.equal(B.grad, pam.matmul(A.detach().T, delta))
+    g = np.load(GOLDEN / "matmul_small.npz")
+    assert_same_bits(host(C), f32(g["p20_c"]).reshape(5, 3), "reference 5x4 @ 4x3 forward")
+    assert np.allclose(host(A.grad), f32(g["p20_da_approx"]).reshape(5, 4)) and np.allclose(host(B.grad), f32(g["p20_db_approx"]).reshape(4, 3))
