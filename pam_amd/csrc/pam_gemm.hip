@@ -379,6 +379,9 @@ int cu_count()
 
 struct Plan { int big; int ksplit; int kchunk; };
 
+// Tuning override for experiments: tile 0 = automatic, 1 = 64x64, 2 = 128x128; ksplit 0 = automatic.
+int g_force_tile = 0, g_force_ksplit = 0;
+
 // Tile shape and split-K factor for a problem.  128x128 tiles (8x8 per lane) when they
 // fill the device, 64x64 (4x4 per lane) otherwise; K is split when even the small tiles
 // leave most compute units idle and K is long.
@@ -388,10 +391,16 @@ Plan make_plan(long batch, long M, long N, long K, bool allow_split)
     auto tiles = [&](long bm, long bn) { return batch * ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     Plan p{0, 1, (int)((K + BK - 1) / BK * BK)};
     if (p.kchunk == 0) p.kchunk = BK;
-    if (tiles(128, 128) >= 2 * cus) { p.big = 1; return p; }
+    if (g_force_tile == 2 || (g_force_tile == 0 && tiles(128, 128) >= 2 * cus)) { p.big = 1; return p; }
     long t = tiles(64, 64);
     long ktiles = (K + BK - 1) / BK;
-    if (allow_split && t < 2 * cus && ktiles >= 16) {
+    if (allow_split && g_force_ksplit > 1) {
+        long per = (ktiles + g_force_ksplit - 1) / g_force_ksplit;
+        p.kchunk = (int)(per * BK);
+        p.ksplit = (int)((ktiles + per - 1) / per);
+        return p;
+    }
+    if (allow_split && g_force_ksplit == 0 && t < 2 * cus && ktiles >= 16) {
         long want = (4 * cus + t - 1) / t;                  // aim at ~4 work-groups per compute unit
         long maxsplit = ktiles / 8;                        // at least 8 k-tiles (128 k) per chunk
         long s = want < maxsplit ? want : maxsplit;
@@ -493,6 +502,8 @@ size_t pam_hip_gemm_workspace_bytes(long batch, long m, long n, long k)
     Plan p = make_plan(batch, m, n, k, true);
     return p.ksplit > 1 ? (size_t)p.ksplit * batch * m * n * sizeof(float) : 0;
 }
+
+void pam_hip_set_tuning(int tile, int ksplit) { g_force_tile = tile; g_force_ksplit = ksplit; }
 
 int pam_hip_gemm_plan(long batch, long m, long n, long k, int* k_splits, int* k_chunk)
 {
