@@ -81,12 +81,14 @@ int pam_hip_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, flo
  * and simply disables that path. */
 size_t pam_hip_gemm_workspace_bytes(long batch, long m, long n, long k);
 
-/* The accumulation order a product of this shape uses when the workspace is supplied:
- * *k_chunk consecutive k are summed in ascending order from +0 into one accumulator per
- * output; with *k_splits > 1 the chunk sums are then added in ascending chunk order, again
- * from +0.  Without a workspace the order is always one chunk (plain ascending k), which is
- * the order of the reference kernel (pam/cuda_kernels.cu:601, 608-627). */
-int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_splits, int *k_chunk);
+/* The accumulation order a product of this shape uses when the workspace is supplied.
+ * k is cut into chunks of *k_chunk consecutive values (a multiple of 16; the last chunk may
+ * be shorter).  Each chunk is summed in ascending k from +0 into one fp32 accumulator per
+ * output.  Every *k_group consecutive chunk sums are added in ascending order, and those
+ * group sums are added in ascending order from +0.  One chunk (k_chunk >= k) is the order
+ * of the reference kernel (pam/cuda_kernels.cu:601, 608-627).  Without a workspace the
+ * order is a single group of *k_group chunks of ceil(ceil(k/16) / k_group) * 16. */
+int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_chunk, int *k_group);
 
 /* Y[m,n] = sum_k A[m,k] (*) B[k,n]            replaces pam_matmul_fwd (matmul_caller<&pam,false>, :703-718) */
 int pam_hip_pam_matmul_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,

@@ -337,9 +337,10 @@ void pamo_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, float
  *         (operand roles pam/cuda_kernels.cu:795-809)
  *
  * Accumulation: fp32, k ascending into one accumulator that starts at +0
- * (pam/cuda_kernels.cu:601).  kchunk > 0 selects the split-K order: every chunk of
- * kchunk consecutive k is summed that way from +0 and the chunk sums are then added
- * in ascending chunk order, again from +0.
+ * (pam/cuda_kernels.cu:601).  kchunk > 0 selects a split order: every chunk of kchunk
+ * consecutive k is summed that way from +0; every kgroup consecutive chunk sums are added in
+ * ascending order (the first one is the starting value); the group sums are then added in
+ * ascending order from +0.
  * Strides are in elements: (batch, row, col) per operand.
  */
 void pamo_gemm(int mode, long batch, long M, long N, long K,
@@ -347,9 +348,10 @@ void pamo_gemm(int mode, long batch, long M, long N, long K,
                const float *R, long rb, long rr, long rc,
                const float *D, long db, long dr, long dc,
                float *Y, long yb, long yr, long yc,
-               float off, long kchunk)
+               float off, long kchunk, long kgroup)
 {
     if (kchunk <= 0 || kchunk > K) kchunk = K > 0 ? K : 1;
+    if (kgroup <= 0) kgroup = 1;
     _Pragma("omp parallel for collapse(2) schedule(static)")
     for (long b = 0; b < batch; b++)
         for (long i = 0; i < M; i++) {
@@ -357,8 +359,9 @@ void pamo_gemm(int mode, long batch, long M, long N, long K,
             for (long j = 0; j < N; j++) {
                 const float *Rp = R + b * rb + j * rc;
                 float d = (mode >= 2) ? D[b * db + i * dr + j * dc] : 0.0f;
-                volatile float total = 0.0f;
-                for (long k0 = 0; k0 < K; k0 += kchunk) {
+                volatile float total = 0.0f, group = 0.0f;
+                long nchunk = 0;
+                for (long k0 = 0; k0 < K || k0 == 0; k0 += kchunk) {
                     long k1 = k0 + kchunk < K ? k0 + kchunk : K;
                     volatile float acc = 0.0f;
                     for (long k = k0; k < k1; k++) {
@@ -371,7 +374,10 @@ void pamo_gemm(int mode, long batch, long M, long N, long K,
                         }
                         acc = acc + p;
                     }
-                    if (kchunk >= K) total = acc; else total = total + acc;
+                    group = (nchunk % kgroup == 0) ? acc : group + acc;
+                    nchunk++;
+                    if (nchunk % kgroup == 0 || k1 >= K) total = total + group;
+                    if (K == 0) break;
                 }
                 Y[b * yb + i * yr + j * yc] = total;
             }

@@ -53,7 +53,7 @@ def lib():
         cl = ctypes.c_long
         L.pamo_gemm.argtypes = [ctypes.c_int, cl, cl, cl, cl,
                                 _fp, cl, cl, cl, _fp, cl, cl, cl, _fp, cl, cl, cl, _fp, cl, cl, cl,
-                                ctypes.c_float, cl]
+                                ctypes.c_float, cl, cl]
         L.pamo_gemm.restype = None
         L.pamo_gemm_fast.argtypes = [cl, cl, cl, _fp, _fp, _fp]
         L.pamo_gemm_fast.restype = None
@@ -175,7 +175,7 @@ def _strides3(a):
     return (0, s[0], s[1]) if a.ndim == 2 else tuple(s)
 
 
-def gemm(L, R, mode=MODE_PAM, D=None, offset=None, kchunk=0):
+def gemm(L, R, mode=MODE_PAM, D=None, offset=None, kchunk=0, kgroup=1):
     """Y = L (x) R for 2-D or 3-D (batched) float32 arrays of any strides."""
     L = np.asarray(L, dtype=np.float32); R = np.asarray(R, dtype=np.float32)
     batched = L.ndim == 3
@@ -189,7 +189,7 @@ def gemm(L, R, mode=MODE_PAM, D=None, offset=None, kchunk=0):
         D = np.asarray(D, dtype=np.float32)
     lib().pamo_gemm(mode, batch, M, N, K,
                     _p(L), *_strides3(L), _p(R), *_strides3(R), _p(D), *_strides3(D),
-                    _p(Y), *_strides3(Y), _off(offset), kchunk)
+                    _p(Y), *_strides3(Y), _off(offset), kchunk, kgroup)
     return Y
 
 

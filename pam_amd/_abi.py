@@ -90,10 +90,10 @@ def device_info():
 
 
 def gemm_plan(batch, m, n, k):
-    """(k_splits, k_chunk): the accumulation order used for this shape."""
-    s, c = _i(0), _i(0)
-    _call("pam_hip_gemm_plan", batch, m, n, k, ctypes.byref(s), ctypes.byref(c))
-    return s.value, c.value
+    """(k_chunk, k_group): the fixed accumulation order used for this shape (see include/pam_hip.h)."""
+    c, g = _i(0), _i(0)
+    _call("pam_hip_gemm_plan", batch, m, n, k, ctypes.byref(c), ctypes.byref(g))
+    return c.value, g.value
 
 
 def _stream():

@@ -4,31 +4,38 @@
 // so the matrix cores do not apply; this is a VALU kernel whose inner loop is, per
 // multiply-accumulate, one v_add_u32 and one v_add_f32.
 //
-//  * A work-group owns a BM x BN tile of Y.  Each lane owns a TM x TN micro-tile in
-//    registers, split into 4-wide groups spread over the tile so that the 128-bit LDS
-//    reads of a wavefront are contiguous (R fragment) or broadcast (L fragment).
-//  * L and R tiles are staged through LDS k-major ([k][row]) with a 4-word row pad, so a
-//    fragment for one k is TM/4 + TN/4 ds_read_b128.  Operands whose contiguous dimension
-//    is k (row-major L, "column-major" R) are transposed on the way in; operands whose
-//    contiguous dimension is the row are stored with 128-bit writes; anything else goes
-//    through a scalar loader.  No transposed copies are made in global memory, so the
-//    backward products run on the views the autograd layer hands over
+//  * A work-group of four wavefronts owns a 64 x 64 tile of Y.  Each lane owns a 4 x 4
+//    micro-tile in registers, each wavefront 32 x 32 outputs (lanes 8 x 8).  Measured on
+//    MI355X, a SIMD retires a wave64 VALU instruction every two cycles but one wavefront
+//    issues at most one every four, so the design goal is many resident wavefronts (five
+//    per SIMD at under 100 registers) rather than a large micro-tile; thousands of equal
+//    work-groups per product are what balances the 256 compute units.
+//  * L and R tiles are staged through LDS k-major ([k][row], 4-word row pad), so a fragment
+//    for one k is two ds_read_b128, contiguous (R) or broadcast (L) across the wavefront.
+//    Operands whose contiguous dimension is k (row-major L, "column-major" R) are
+//    transposed on the way in; operands contiguous along the row use 128-bit LDS writes;
+//    anything else goes through a scalar loader.  No transposed copies are made in global
+//    memory, so the backward products run on the views the autograd layer hands over
 //    (pam/cuda_bindings.py:147-164).
-//  * Global loads for tile t+1 are issued before the arithmetic of tile t (register
-//    double buffering), LDS is double buffered, one barrier per k-tile.
+//  * Global loads for k-tile t+1 are issued before the arithmetic of tile t (register
+//    double buffering), LDS is double buffered, one barrier per k-tile.  k-tiles are 32
+//    deep for long k and 16 deep for short k.
 //  * The bias subtraction and the optional offset (R' = R (*) offset) are applied once per
 //    element while staging R.
-//  * While staging, every element is classified: if all of a k-tile's L and R values are
-//    normal numbers with magnitude in [2^-63, 2^64), no product in the tile can leave the
-//    normal range and the two-instruction loop is exact.  Otherwise (zeros, subnormals,
-//    inf, NaN, extreme exponents) the work-group takes a guarded loop for that k-tile,
-//    which evaluates the full definition per product.  The choice is uniform per
-//    work-group and per k-tile.
+//  * While staging, every element's exponent is folded into a running min/max.  If all of a
+//    k-tile's L and R values are normal numbers with magnitude in [2^-63, 2^64), no product
+//    in the tile can leave the normal range and the two-instruction loop is exact;
+//    otherwise (zeros, subnormals, inf, NaN, extreme exponents) the work-group takes a
+//    guarded loop for that k-tile, which evaluates the full definition per product on
+//    operands decomposed once per k-step.  The choice is uniform per work-group and k-tile.
 //  * Rows beyond M / N are clamped to the last valid row when loading (their results are
 //    never stored); the k tail runs a shorter loop, padding never enters the arithmetic.
-//  * Accumulation order: every output is summed by one lane, k ascending, from +0 -- the
-//    order of the reference kernel (pam/cuda_kernels.cu:601, 608-627).  With split-K the
-//    chunk sums are added in ascending chunk order by a second kernel.
+//  * Shapes with few output tiles and long k (dX: 12608 x 192, k = 768; dW: 192 x 768,
+//    k = 12608) split k across work-groups; the partial tiles go through a scratch buffer
+//    and are added in ascending order by a second kernel.
+//  * Accumulation order: every output is summed by one lane per k chunk, k ascending, from
+//    +0 -- with one chunk this is the order of the reference kernel
+//    (pam/cuda_kernels.cu:601, 608-627); pam_hip_gemm_plan reports the chunking.
 #include "pam_common.h"
 #include "pam_device.h"
 
@@ -39,7 +46,7 @@ namespace {
 enum { MODE_PAM = 0, MODE_STD = 1, MODE_BWD_DL = 2, MODE_BWD_DR = 3 };
 enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2 };   // k contiguous / row contiguous / any strides
 
-constexpr int BK = 16;
+constexpr int KGRAN = 32;         // k ranges handed to work-groups are multiples of this
 constexpr int PAD = 4;
 
 struct Operand { const float* p; long sb, sr, sk; };    // batch, row (the non-k index), k strides
@@ -48,43 +55,38 @@ struct GemmArgs {
     const float* D; long d_sb, d_sr, d_sc;
     float* Y; long y_sb, y_sr, y_sc;
     int M, N, K;
-    int ksplit, kchunk;          // kchunk is a multiple of BK; ksplit == 1 means no split
+    int ksplit, kchunk;          // kchunk is a multiple of 32; ksplit == 1 means no split
     float off; int has_off;
 };
 
-// magnitude in [2^-63, 2^64): exponent field 64 .. 190
-__device__ __forceinline__ bool in_window(uint32_t u) { return ((u >> 23) & 0xffu) - 64u < 127u; }
-
+// Classifies and transforms one staged value.  MODE_PAM: R carries the bias subtraction.
+// Backward modes: the "slope side" is the forward operand b of pam_bwd(a, b, delta).
 template <int MODE, bool IS_R>
-__device__ __forceinline__ uint32_t stage_value(float v, float off, bool has_off, bool& bad)
-{
-    // which operand carries exponent information ("b" of pam_bwd) in the backward modes
-    constexpr bool kIsSlopeSide = (MODE == MODE_BWD_DL && IS_R) || (MODE == MODE_BWD_DR && !IS_R);
-    if (MODE == MODE_STD) return f2u(v);
-    if (MODE == MODE_PAM) {
-        if (IS_R) {
-            if (has_off) v = pam_mul(v, off);
-            uint32_t u = f2u(v);
-            bad |= !in_window(u);
-            return u - kBias;
+struct Stager {
+    static constexpr bool kSlopeSide = (MODE == MODE_BWD_DL && IS_R) || (MODE == MODE_BWD_DR && !IS_R);
+    static constexpr bool kDeltaSide = (MODE >= MODE_BWD_DL) && !kSlopeSide;
+    static constexpr bool kTakesOffset = (MODE == MODE_PAM && IS_R) || kSlopeSide;
+    uint32_t emin = 255u, emax = 0u;
+    bool bad = false;
+
+    __device__ __forceinline__ uint32_t one(float v)
+    {
+        uint32_t u = f2u(v);
+        if (MODE == MODE_STD) return u;
+        if (kDeltaSide) {                          // the upstream gradient: zero is harmless
+            bad |= !((((u >> 23) & 0xffu) - 64u < 127u) || (u & ~kSign) == 0);
+            return u;
         }
-        uint32_t u = f2u(v);
-        bad |= !in_window(u);
-        return u;
+        uint32_t e = (u >> 23) & 0xffu;
+        emin = min(emin, e); emax = max(emax, e);
+        return (MODE == MODE_PAM && IS_R) ? u - kBias : u;
     }
-    if (kIsSlopeSide) {
-        if (has_off) v = pam_mul(v, off);
-        uint32_t u = f2u(v);
-        bad |= !in_window(u);
-        return u;
-    }
-    uint32_t u = f2u(v);                        // the upstream gradient: zero is harmless
-    bad |= !(in_window(u) || (u & ~kSign) == 0);
-    return u;
-}
+    // true when some staged value lies outside [2^-63, 2^64) or is not a normal number
+    __device__ __forceinline__ bool guarded() const { return bad || emin < 64u || emax > 190u; }
+};
 
 // One operand's tile: ROWS x BK values from global memory into registers, then into LDS.
-template <int ROWS, int NT, int KIND>
+template <int ROWS, int NT, int KIND, int BK>
 struct TileLoader {
     static constexpr int kVecs = ROWS * BK / 4 / NT;      // float4 per lane (vector kinds)
     static constexpr int kElems = ROWS * BK / NT;         // scalars per lane (generic kind)
@@ -124,43 +126,75 @@ struct TileLoader {
         }
     }
 
-    template <int MODE, bool IS_R>
-    __device__ __forceinline__ void store(uint32_t* lds, int tid, float off, bool has_off, bool& bad)
+    // R' = R (*) offset, once per element (uniform branch around the whole tile)
+    __device__ __forceinline__ void apply_offset(float off)
+    {
+        float* s = reinterpret_cast<float*>(v);
+#pragma unroll 1
+        for (int i = 0; i < kElems; ++i) s[i] = pam_mul(s[i], off);
+    }
+
+    template <class S>
+    __device__ __forceinline__ void store(uint32_t* lds, int tid, S& st)
     {
         constexpr int LD = ROWS + PAD;
         if (KIND == LOAD_KVEC) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
-                int r = id / (BK / 4), kq = id % (BK / 4);
-                lds[(kq * 4 + 0) * LD + r] = stage_value<MODE, IS_R>(v[i].x, off, has_off, bad);
-                lds[(kq * 4 + 1) * LD + r] = stage_value<MODE, IS_R>(v[i].y, off, has_off, bad);
-                lds[(kq * 4 + 2) * LD + r] = stage_value<MODE, IS_R>(v[i].z, off, has_off, bad);
-                lds[(kq * 4 + 3) * LD + r] = stage_value<MODE, IS_R>(v[i].w, off, has_off, bad);
+                uint32_t* d = lds + ((id % (BK / 4)) * 4) * LD + id / (BK / 4);
+                d[0 * LD] = st.one(v[i].x); d[1 * LD] = st.one(v[i].y);
+                d[2 * LD] = st.one(v[i].z); d[3 * LD] = st.one(v[i].w);
             }
         } else if (KIND == LOAD_RVEC) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
-                int k = id / (ROWS / 4), rq = id % (ROWS / 4);
                 uint4 w;
-                w.x = stage_value<MODE, IS_R>(v[i].x, off, has_off, bad);
-                w.y = stage_value<MODE, IS_R>(v[i].y, off, has_off, bad);
-                w.z = stage_value<MODE, IS_R>(v[i].z, off, has_off, bad);
-                w.w = stage_value<MODE, IS_R>(v[i].w, off, has_off, bad);
-                *reinterpret_cast<uint4*>(lds + k * LD + rq * 4) = w;
+                w.x = st.one(v[i].x); w.y = st.one(v[i].y); w.z = st.one(v[i].z); w.w = st.one(v[i].w);
+                *reinterpret_cast<uint4*>(lds + (id / (ROWS / 4)) * LD + (id % (ROWS / 4)) * 4) = w;
             }
         } else {
             const float* s = reinterpret_cast<const float*>(v);
 #pragma unroll
             for (int i = 0; i < kElems; ++i) {
                 int id = tid + i * NT;
-                int k = id / ROWS, r = id % ROWS;
-                lds[k * LD + r] = stage_value<MODE, IS_R>(s[i], off, has_off, bad);
+                lds[(id / ROWS) * LD + id % ROWS] = st.one(s[i]);
             }
         }
     }
 };
+
+// Guarded PAM product on decomposed operands.  An operand is split once per k-step into
+//   ex = unbiased exponent (+127 folded into the L side), or a sentinel: -2^12 for zero,
+//        +2^20 for inf/NaN;
+//   fr = 23-bit fraction with subnormals normalised, the sign in bit 31 (cleared for zeros,
+//        whose sign the reference's float emulation ignores, pam/native.py:54).
+// A pair then costs two adds and a range check; zeros fall out of the underflow branch with
+// the sign of the other operand, inf/NaN out of the overflow branch.
+struct Split { int ex; uint32_t fr; };
+
+__device__ __forceinline__ Split split_operand(uint32_t u, int bias)
+{
+    uint32_t mag = u & ~kSign;
+    Split s;
+    if (__builtin_expect(mag - 0x00800000u < 0x7f000000u, 1)) {
+        s.ex = (int)(mag >> 23) - 127 + bias; s.fr = u & (kSign | kMant);
+    } else if (mag == 0) { s.ex = -4096; s.fr = 0; }
+    else if (mag >= kExpo) { s.ex = 1 << 20; s.fr = 0; }
+    else { int e; uint32_t m; split_mag(mag, e, m); s.ex = e + bias; s.fr = (u & kSign) | m; }
+    return s;
+}
+
+__device__ __forceinline__ float guarded_product(const Split& a, const Split& b)
+{
+    uint32_t f = a.fr + b.fr;                        // bit 31: sign, bit 23: fraction carry
+    int eb = a.ex + b.ex + (int)((f >> 23) & 1u);    // biased exponent of the product
+    uint32_t sign = f & kSign, frac = f & kMant;
+    if (__builtin_expect((uint32_t)(eb - 1) < 254u, 1)) return u2f(sign | ((uint32_t)eb << 23) | frac);
+    if (eb > (1 << 19)) return u2f(kQNaN);           // an inf/NaN operand
+    return u2f(join_mag(sign, eb - 127, frac));      // overflow, gradual underflow, zero
+}
 
 // Exact-backward product from the normalised mantissa fraction of the forward operand
 // whose gradient is wanted, the other forward operand b (offset already applied) and the
@@ -189,7 +223,7 @@ __device__ __forceinline__ uint32_t normalised_fraction(float d)
     return m;
 }
 
-template <int BM, int BN, int TM, int TN, int MODE, int LKIND, int RKIND>
+template <int BM, int BN, int TM, int TN, int BK, int MODE, int LKIND, int RKIND>
 __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g, float* __restrict__ partial)
 {
     constexpr int TXN = BN / TN, TYN = BM / TM, NT = TXN * TYN, NW = NT / 64;
@@ -203,8 +237,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
 
     const int tid = threadIdx.x, tx = tid % TXN, ty = tid / TXN;
     const int wave = tid / 64, lane = tid % 64;
-    const int zb = blockIdx.z / g.ksplit, zs = blockIdx.z % g.ksplit;
-    const int row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
+    const int zb = blockIdx.z, zs = blockIdx.y;
+    const int ntn = (g.N + BN - 1) / BN;                  // consecutive work-groups share L rows
+    const int row0 = (blockIdx.x / ntn) * BM, col0 = (blockIdx.x % ntn) * BN;
     const int kbegin = zs * g.kchunk;
     const int kend = min(g.K, kbegin + g.kchunk);
     const int ktiles = (kend - kbegin + BK - 1) / BK;
@@ -233,15 +268,19 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
             }
     }
 
-    TileLoader<BM, NT, LKIND> ll;
-    TileLoader<BN, NT, RKIND> rl;
+    TileLoader<BM, NT, LKIND, BK> ll;
+    TileLoader<BN, NT, RKIND, BK> rl;
 
     auto stage = [&](int buf) {
-        bool bad = false;
-        ll.template store<MODE, false>(lds_l[buf], tid, g.off, has_off, bad);
-        rl.template store<MODE, true>(lds_r[buf], tid, g.off, has_off, bad);
+        Stager<MODE, false> sl; Stager<MODE, true> sr;
+        if (has_off) {
+            if (Stager<MODE, false>::kTakesOffset) ll.apply_offset(g.off);
+            if (Stager<MODE, true>::kTakesOffset) rl.apply_offset(g.off);
+        }
+        ll.store(lds_l[buf], tid, sl);
+        rl.store(lds_r[buf], tid, sr);
         if (MODE != MODE_STD) {
-            unsigned long long any = __ballot(bad);
+            unsigned long long any = __ballot(sl.guarded() || sr.guarded());
             if (lane == 0) lds_flag[buf][wave] = any != 0ull;
         }
     };
@@ -299,12 +338,23 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
         auto guarded_step = [&](int kk) {
             uint32_t a[TM], b[TN];
             fragment(kk, a, b);
+            if (MODE == MODE_PAM) {
+                Split sa[TM], sb[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) sa[i] = split_operand(a[i], 127);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) sb[j] = split_operand(b[j] + kBias, 0);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] += guarded_product(sa[i], sb[j]);
+                return;
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
-                    if (MODE == MODE_PAM) acc[i][j] += pam_mul(u2f(a[i]), u2f(b[j] + kBias));
-                    else if (MODE == MODE_BWD_DL) acc[i][j] += bwd_product_general(dfrac[i][j], b[j], u2f(a[i]));
+                    if (MODE == MODE_BWD_DL) acc[i][j] += bwd_product_general(dfrac[i][j], b[j], u2f(a[i]));
                     else if (MODE == MODE_BWD_DR) acc[i][j] += bwd_product_general(dfrac[i][j], a[i], u2f(b[j]));
                 }
         };
@@ -329,7 +379,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
     // epilogue: to Y, or to this chunk's slab of the split-K scratch ([chunk][batch][M][N])
     float* out; long o_sr, o_sc;
     if (g.ksplit > 1) {
-        out = partial + ((long)zs * (gridDim.z / g.ksplit) + zb) * (long)g.M * g.N; o_sr = g.N; o_sc = 1;
+        out = partial + ((long)zs * gridDim.z + zb) * (long)g.M * g.N; o_sr = g.N; o_sc = 1;
     } else {
         out = g.Y + (long)zb * g.y_sb; o_sr = g.y_sr; o_sc = g.y_sc;
     }
@@ -377,38 +427,31 @@ int cu_count()
     return g_cus;
 }
 
-struct Plan { int big; int ksplit; int kchunk; };
+struct Plan { int bk; int ksplit; int kchunk; };
 
-// Tuning override for experiments: tile 0 = automatic, 1 = 64x64, 2 = 128x128; ksplit 0 = automatic.
-int g_force_tile = 0, g_force_ksplit = 0;
+// Tuning override for experiments: bk 0 = automatic (16 or 32), ksplit 0 = automatic.
+int g_force_bk = 0, g_force_ksplit = 0;
 
-// Tile shape and split-K factor for a problem.  128x128 tiles (8x8 per lane) when they
-// fill the device, 64x64 (4x4 per lane) otherwise; K is split when even the small tiles
-// leave most compute units idle and K is long.
+// Work-groups own 64 x 64 output tiles.  Long k uses 32-deep k-tiles (fewer barriers and
+// more bytes in flight per round), short k 16-deep ones.  k is split across work-groups
+// when the tiles alone do not give each compute unit several work-groups: the aim is about
+// eight equal work-groups per unit, each at least 128 deep in k.
 Plan make_plan(long batch, long M, long N, long K, bool allow_split)
 {
     const long cus = cu_count();
-    auto tiles = [&](long bm, long bn) { return batch * ((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    Plan p{0, 1, (int)((K + BK - 1) / BK * BK)};
-    if (p.kchunk == 0) p.kchunk = BK;
-    if (g_force_tile == 2 || (g_force_tile == 0 && tiles(128, 128) >= 2 * cus)) { p.big = 1; return p; }
-    long t = tiles(64, 64);
-    long ktiles = (K + BK - 1) / BK;
-    if (allow_split && g_force_ksplit > 1) {
-        long per = (ktiles + g_force_ksplit - 1) / g_force_ksplit;
-        p.kchunk = (int)(per * BK);
-        p.ksplit = (int)((ktiles + per - 1) / per);
-        return p;
-    }
-    if (allow_split && g_force_ksplit == 0 && t < 2 * cus && ktiles >= 16) {
-        long want = (4 * cus + t - 1) / t;                  // aim at ~4 work-groups per compute unit
-        long maxsplit = ktiles / 8;                        // at least 8 k-tiles (128 k) per chunk
-        long s = want < maxsplit ? want : maxsplit;
-        if (s > 1) {
-            long per = (ktiles + s - 1) / s;
-            p.kchunk = (int)(per * BK);
-            p.ksplit = (int)((ktiles + per - 1) / per);
-        }
+    const long tiles = batch * ((M + 63) / 64) * ((N + 63) / 64);
+    const long kunits = K > 0 ? (K + KGRAN - 1) / KGRAN : 1;
+    Plan p{K >= 512 ? 32 : 16, 1, (int)(kunits * KGRAN)};
+    if (g_force_bk) p.bk = g_force_bk;
+    long want = 1;
+    if (g_force_ksplit > 0) want = g_force_ksplit;
+    else if (tiles < 6 * cus) want = (8 * cus + tiles - 1) / tiles;
+    long maxsplit = kunits / 4;                                  // at least 128 k per work-group
+    if (want > maxsplit) want = maxsplit;
+    if (allow_split && want > 1) {
+        long per = (kunits + want - 1) / want;
+        p.kchunk = (int)(per * KGRAN);
+        p.ksplit = (int)((kunits + per - 1) / per);
     }
     return p;
 }
@@ -421,12 +464,11 @@ int load_kind(long s_row, long s_k, long s_batch, const float* p, long rows, lon
     return LOAD_ANY;
 }
 
-template <int BM, int BN, int TM, int TN, int MODE>
+template <int BK, int MODE>
 void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, float* partial)
 {
-    constexpr int NT = (BM / TM) * (BN / TN);
 #define PAM_GEMM_CASE(LK, RK) \
-    if (lk == LK && rk == RK) { hipLaunchKernelGGL((gemm_kernel<BM, BN, TM, TN, MODE, LK, RK>), grid, dim3(NT), 0, st, g, partial); return; }
+    if (lk == LK && rk == RK) { hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 4, BK, MODE, LK, RK>), grid, dim3(256), 0, st, g, partial); return; }
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
@@ -436,13 +478,9 @@ void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, 
 template <int MODE>
 void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& g, long batch, float* partial)
 {
-    if (p.big) {
-        dim3 grid((g.N + 127) / 128, (g.M + 127) / 128, (unsigned)(batch * p.ksplit));
-        launch_kinds<128, 128, 8, 8, MODE>(lk, rk, grid, st, g, partial);
-    } else {
-        dim3 grid((g.N + 63) / 64, (g.M + 63) / 64, (unsigned)(batch * p.ksplit));
-        launch_kinds<64, 64, 4, 4, MODE>(lk, rk, grid, st, g, partial);
-    }
+    dim3 grid((unsigned)(((g.N + 63) / 64) * (long)((g.M + 63) / 64)), (unsigned)p.ksplit, (unsigned)batch);
+    if (p.bk == 32) launch_kinds<32, MODE>(lk, rk, grid, st, g, partial);
+    else launch_kinds<16, MODE>(lk, rk, grid, st, g, partial);
 }
 
 int gemm(const char* what, int mode, long batch, long M, long N, long K,
@@ -453,18 +491,15 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     if (batch < 0 || M < 0 || N < 0 || K < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: negative size", what);
     if (batch == 0 || M == 0 || N == 0) return PAM_HIP_OK;
     if (!l || !r || !y || (mode >= MODE_BWD_DL && !d)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: null pointer", what);
-    if (M > 0x7ffffff0L || N > 0x7ffffff0L || K > 0x7ffffff0L)
-        return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: dimension beyond 2^31", what);
+    if (M > (1L << 30) || N > (1L << 30) || K > (1L << 30) || batch > 65535 || ((M + 63) / 64) * ((N + 63) / 64) > 0x7fffffffL)
+        return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: dimension too large (sizes <= 2^30, batch <= 65535, output tiles < 2^31)", what);
     hipStream_t st = (hipStream_t)stream;
 
     Plan p = make_plan(batch, M, N, K, workspace != nullptr);
-    if (batch * p.ksplit > 65535) { p.ksplit = 1; p.kchunk = (int)((K + BK - 1) / BK * BK); }
-    if (batch > 65535) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: batch beyond 65535", what);
-    if (p.ksplit > 1) {
-        size_t need = (size_t)p.ksplit * batch * M * N * sizeof(float);
-        if (need > workspace_bytes) { p.ksplit = 1; p.kchunk = (int)((K + BK - 1) / BK * BK); }
+    if (p.ksplit > 1 && (size_t)p.ksplit * batch * M * N * sizeof(float) > workspace_bytes) {
+        p.ksplit = 1; p.kchunk = (int)((K + KGRAN - 1) / KGRAN * KGRAN);
     }
-    if (p.kchunk < BK) p.kchunk = BK;
+    if (p.kchunk < KGRAN) p.kchunk = KGRAN;
 
     GemmArgs g;
     g.L = Operand{l, l_sb, l_sr, l_sc};
@@ -503,15 +538,14 @@ size_t pam_hip_gemm_workspace_bytes(long batch, long m, long n, long k)
     return p.ksplit > 1 ? (size_t)p.ksplit * batch * m * n * sizeof(float) : 0;
 }
 
-void pam_hip_set_tuning(int tile, int ksplit) { g_force_tile = tile; g_force_ksplit = ksplit; }
+void pam_hip_set_tuning(int bk, int ksplit) { g_force_bk = bk; g_force_ksplit = ksplit; }
 
-int pam_hip_gemm_plan(long batch, long m, long n, long k, int* k_splits, int* k_chunk)
+int pam_hip_gemm_plan(long batch, long m, long n, long k, int* k_chunk, int* k_group)
 {
     if (batch <= 0 || m <= 0 || n <= 0 || k < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "gemm_plan: bad shape");
     Plan p = make_plan(batch, m, n, k, true);
-    if (batch * p.ksplit > 65535) { p.ksplit = 1; p.kchunk = (int)((k + BK - 1) / BK * BK); }
-    if (k_splits) *k_splits = p.ksplit;
-    if (k_chunk) *k_chunk = p.ksplit > 1 ? p.kchunk : (int)k;
+    if (k_chunk) *k_chunk = p.kchunk;
+    if (k_group) *k_group = 1;
     return PAM_HIP_OK;
 }
 

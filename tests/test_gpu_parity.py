@@ -37,6 +37,16 @@ def host(t):
 OFFS = [None, 1.0552]
 
 
+def ogemm(oracle, L, R, plan_shape=None, **kw):
+    """The oracle's product in the fixed accumulation order the library uses for this shape
+    (plan_shape = (batch, m, n, k) of the full product when L, R are a sample of it)."""
+    from pam_amd import _abi
+    L = np.asarray(L); R = np.asarray(R)
+    batch = L.shape[0] if L.ndim == 3 else 1
+    chunk, group = _abi.gemm_plan(*(plan_shape or (batch, L.shape[-2], R.shape[-1], L.shape[-1])))
+    return oracle.gemm(L, R, kchunk=chunk, kgroup=group, **kw)
+
+
 def _o(off):
     return 1.0 if off is None else off
 
@@ -192,12 +202,12 @@ SHAPES = [(5, 4, 3), (64, 16, 64), (70, 33, 45), (130, 100, 257), (128, 197, 128
 @pytest.mark.parametrize("m,k,n", SHAPES)
 def test_matmul_forward_layouts(K, oracle, m, k, n):
     A, B = _rand((m, k), m + k), _rand((k, n), n + k + 1)
-    want = oracle.gemm(A, B)
+    want = ogemm(oracle, A, B)
     for la, ta in _layouts(A).items():
         for lb, tb in _layouts(B).items():
             assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), want, f"{la} x {lb}")
-    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), oracle.gemm(A, B, offset=1.0552), "offset")
-    assert_same_bits(host(K.standard_matmul(dev(A), dev(B), True, True, 1.0)), oracle.gemm(A, B, mode=oracle.MODE_STD), "standard")
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), ogemm(oracle, A, B, offset=1.0552), "offset")
+    assert_same_bits(host(K.standard_matmul(dev(A), dev(B), True, True, 1.0)), ogemm(oracle, A, B, mode=oracle.MODE_STD), "standard")
 
 
 @pytest.mark.parametrize("zeros,specials", [(0.5, False), (0.02, True), (1.0, False)])
@@ -205,8 +215,8 @@ def test_matmul_zeros_and_specials(K, oracle, zeros, specials):
     A, B = _rand((150, 75), 1, zeros, specials), _rand((75, 90), 2, zeros / 2, specials)
     for la, ta in _layouts(A).items():
         for lb, tb in _layouts(B).items():
-            assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), oracle.gemm(A, B), f"{la} x {lb}")
-    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), oracle.gemm(A, B, offset=1.0552), "offset")
+            assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), ogemm(oracle, A, B), f"{la} x {lb}")
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), ogemm(oracle, A, B, offset=1.0552), "offset")
 
 
 @pytest.mark.parametrize("delta_l", [True, False])
@@ -215,7 +225,7 @@ def test_matmul_exact_backward(K, oracle, delta_l, zeros, specials):
     L, R, D = _rand((70, 45), 3, zeros, specials), _rand((45, 97), 4, zeros, specials), _rand((70, 97), 5, zeros / 3, specials)
     mode = oracle.MODE_BWD_DELTA_L if delta_l else oracle.MODE_BWD_DELTA_R
     for off in OFFS:
-        want = oracle.gemm(L, R, mode=mode, D=D, offset=off)
+        want = ogemm(oracle, L, R, mode=mode, D=D, offset=off)
         for ll, tl in _layouts(L).items():
             for lr, tr in _layouts(R).items():
                 got = host(K.pam_matmul_bwd(tl, tr, dev(D), True, True, delta_l, _o(off)))
@@ -233,32 +243,35 @@ def test_bmm_tails_and_strides(K, oracle):
     Q, Kt = _rand((6, 197, 64), 7), _rand((6, 64, 197), 8)
     P, V = _rand((6, 197, 197), 9, zeros=0.1), _rand((6, 197, 64), 10)
     for L, R in ((Q, Kt), (P, V)):
-        want = oracle.gemm(L, R)
+        want = ogemm(oracle, L, R)
         for ll, tl in _layouts(L).items():
             for lr, tr in _layouts(R).items():
                 assert_same_bits(host(K.pam_bmm_fwd(tl, tr, True, True, 1.0)), want, f"bmm {ll} x {lr}")
     D = _rand((6, 197, 64), 11)
     assert_same_bits(host(K.pam_bmm_bwd(dev(P), dev(V), dev(D), True, True, True, 1.0)),
-                     oracle.gemm(P, V, mode=oracle.MODE_BWD_DELTA_L, D=D), "bmm bwd")
+                     ogemm(oracle, P, V, mode=oracle.MODE_BWD_DELTA_L, D=D), "bmm bwd")
     # fairseq-style strided batch: q = x.view(T, B*H, D).transpose(0, 1), batch stride < row stride
     T, BH, Dh = 32, 12, 16
     x = _rand((T, BH, Dh), 12); y = _rand((T, BH, Dh), 13)
     q = dev(x).transpose(0, 1); kt = dev(y).transpose(0, 1).transpose(1, 2)
     assert q.stride() == (Dh, BH * Dh, 1) and kt.stride() == (Dh, 1, BH * Dh)
-    want = oracle.gemm(np.swapaxes(x, 0, 1), np.swapaxes(np.swapaxes(y, 0, 1), 1, 2))
+    want = ogemm(oracle, np.swapaxes(x, 0, 1), np.swapaxes(np.swapaxes(y, 0, 1), 1, 2))
     assert_same_bits(host(K.pam_bmm_fwd(q, kt, True, False, 1.0)), want, "strided batch")
 
 
 def test_split_k_fixed_order(K, oracle):
     from pam_amd import _abi
-    m, n, k = 96, 160, 4096
-    splits, chunk = _abi.gemm_plan(1, m, n, k)
-    assert splits > 1 and chunk % 16 == 0
+    m, n, k = 96, 160, 8192
+    chunk, group = _abi.gemm_plan(1, m, n, k)
+    assert chunk % 16 == 0 and chunk * group < k, "this shape is expected to split k across work-groups"
     A, B = _rand((m, k), 14), _rand((k, n), 15)
-    want = oracle.gemm(A, B, kchunk=chunk)
+    want = oracle.gemm(A, B, kchunk=chunk, kgroup=group)
     assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)), want, "split-K order")
     At = dev(np.ascontiguousarray(A.T)).T                      # the dW layout: column-major left operand
     assert_same_bits(host(K.pam_matmul_fwd(At, dev(B), False, True, 1.0)), want, "split-K, cm x rm")
+    # the sequential order differs from the split order only by fp32 rounding of the sums
+    seq = oracle.gemm(A, B)
+    assert np.abs(seq - want).max() <= 1e-5 * np.abs(seq).max()
 
 
 def test_matmul_config0_golden(K, oracle):
@@ -266,18 +279,12 @@ def test_matmul_config0_golden(K, oracle):
     g = np.load(GOLDEN / "matmul_c0.npz")
     A, B, dY = c0_operands()
     Y = host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)); want = f32(g["y"]).reshape(256, 256)
-    assert_same_bits(Y, oracle.gemm(A, B, kchunk=_plan_chunk(256, 256, 512)), "config 0 forward vs oracle")
+    assert_same_bits(Y, ogemm(oracle, A, B), "config 0 forward vs oracle")
     assert np.abs(Y - want).max() / np.abs(want).max() <= 1e-5                  # vs native.pam_matmul
     dA = host(K.pam_matmul_fwd(dev(dY), dev(B).T, True, False, 1.0))
     dB = host(K.pam_matmul_fwd(dev(A).T, dev(dY), False, True, 1.0))
     assert np.abs(dA[::8] - f32(g["da_rows"]).reshape(32, 512)).max() / np.abs(f32(g["da_rows"])).max() <= 1e-5
     assert np.abs(dB[::8] - f32(g["db_rows"]).reshape(64, 256)).max() / np.abs(f32(g["db_rows"])).max() <= 1e-5
-
-
-def _plan_chunk(m, n, k, batch=1):
-    from pam_amd import _abi
-    splits, chunk = _abi.gemm_plan(batch, m, n, k)
-    return chunk if splits > 1 else 0
 
 
 # ------------------------------------------------------------------ full-size configurations
@@ -294,10 +301,10 @@ def test_deit_linear_full_size(K, oracle):
     dX = K.pam_matmul_fwd(tdY, tW, True, True, 1.0)
     dW = K.pam_matmul_fwd(tX.T, tdY, False, True, 1.0)
     rows = rng.choice(12608, 48, replace=False)
-    assert_same_bits(host(Y)[rows], oracle.gemm(X[rows], W.T, kchunk=_plan_chunk(12608, 768, 192)), "Y rows")
-    assert_same_bits(host(dX)[rows], oracle.gemm(dY[rows], W, kchunk=_plan_chunk(12608, 192, 768)), "dX rows")
+    assert_same_bits(host(Y)[rows], ogemm(oracle, X[rows], W.T, plan_shape=(1, 12608, 768, 192)), "Y rows")
+    assert_same_bits(host(dX)[rows], ogemm(oracle, dY[rows], W, plan_shape=(1, 12608, 192, 768)), "dX rows")
     cols = rng.choice(768, 24, replace=False)
-    assert_same_bits(host(dW)[:, cols], oracle.gemm(X.T, dY[:, cols], kchunk=_plan_chunk(192, 768, 12608)), "dW cols")
+    assert_same_bits(host(dW)[:, cols], ogemm(oracle, X.T, dY[:, cols], plan_shape=(1, 192, 768, 12608)), "dW cols")
     # multiplying an operand by a power of two multiplies every PAM product, hence the sum, exactly
     assert torch.equal(K.pam_matmul_fwd(tX * 4.0, tW.T, True, False, 1.0), Y * 4.0)
     assert torch.equal(K.pam_matmul_fwd(tX, (tW * 0.5).T, True, False, 1.0), Y * 0.5)
@@ -342,13 +349,13 @@ def test_linear_autograd_matches_oracle(K, oracle):
         x = dev(X).requires_grad_()
         y = lin(x); y.backward(dev(dY))
         X2, dY2 = X.reshape(200, 96), dY.reshape(200, 40)
-        assert_same_bits(host(y).reshape(200, 40), oracle.gemm(X2, W.T) + bias, "linear forward")
+        assert_same_bits(host(y).reshape(200, 40), ogemm(oracle, X2, W.T) + bias, "linear forward")
         if approx:
-            assert_same_bits(host(x.grad).reshape(200, 96), oracle.gemm(dY2, W), "dX approx")
-            assert_same_bits(host(lin.weight.grad), oracle.gemm(X2.T, dY2).T, "dW approx")
+            assert_same_bits(host(x.grad).reshape(200, 96), ogemm(oracle, dY2, W), "dX approx")
+            assert_same_bits(host(lin.weight.grad), ogemm(oracle, X2.T, dY2).T, "dW approx")
         else:
-            assert_same_bits(host(x.grad).reshape(200, 96), oracle.gemm(dY2, W, mode=oracle.MODE_BWD_DELTA_L, D=X2), "dX exact")
-            assert_same_bits(host(lin.weight.grad), oracle.gemm(X2.T, dY2, mode=oracle.MODE_BWD_DELTA_R, D=W.T).T, "dW exact")
+            assert_same_bits(host(x.grad).reshape(200, 96), ogemm(oracle, dY2, W, mode=oracle.MODE_BWD_DELTA_L, D=X2), "dX exact")
+            assert_same_bits(host(lin.weight.grad), ogemm(oracle, X2.T, dY2, mode=oracle.MODE_BWD_DELTA_R, D=W.T).T, "dW exact")
 
 
 def test_reference_vectors_on_device(K):
