@@ -48,20 +48,51 @@ __device__ __forceinline__ uint32_t join_mag(uint32_t sign, int E, uint32_t M)
     return sign | q;
 }
 
-__device__ __noinline__ float pam_general(uint32_t ai, uint32_t bi)
+// An operand decomposed for the general (any class) product and quotient:
+//   ex = unbiased exponent plus `bias`, or a sentinel: -4096 for zero, +2^20 for inf/NaN;
+//   fr = 23-bit fraction with subnormals normalised, the sign in bit 31 (cleared for zeros,
+//        whose sign the reference's float emulation ignores, pam/native.py:54, 163).
+struct Split { int ex; uint32_t fr; };
+
+__device__ __forceinline__ Split split_operand(uint32_t u, int bias)
 {
-    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
-    if (ma >= kExpo || mb >= kExpo) return u2f(kQNaN);
-    if (ma == 0 || mb == 0) {
-        uint32_t s = (ma ? ai : 0u) ^ (mb ? bi : 0u);
-        return u2f(s & kSign);
-    }
-    int ea, eb; uint32_t fa, fb;
-    split_mag(ma, ea, fa); split_mag(mb, eb, fb);
-    uint32_t M = fa + fb; int E = ea + eb;
-    if (M & 0x00800000u) { E += 1; M &= kMant; }
-    return u2f(join_mag((ai ^ bi) & kSign, E, M));
+    uint32_t mag = u & ~kSign;
+    Split s;
+    if (__builtin_expect(mag - 0x00800000u < 0x7f000000u, 1)) {
+        s.ex = (int)(mag >> 23) - 127 + bias; s.fr = u & (kSign | kMant);
+    } else if (mag == 0) { s.ex = -4096; s.fr = 0; }
+    else if (mag >= kExpo) { s.ex = 1 << 20; s.fr = 0; }
+    else { int e; uint32_t m; split_mag(mag, e, m); s.ex = e + bias; s.fr = (u & kSign) | m; }
+    return s;
 }
+
+// Product of decomposed operands whose biases add up to 127.  Zeros fall out of the
+// underflow branch with the sign of the other operand, inf/NaN out of the overflow branch.
+__device__ __forceinline__ float pam_from_split(const Split& a, const Split& b)
+{
+    uint32_t f = a.fr + b.fr;                        // bit 31: sign, bit 23: fraction carry
+    int eb = a.ex + b.ex + (int)((f >> 23) & 1u);    // biased exponent of the product
+    uint32_t sign = f & kSign, frac = f & kMant;
+    if (__builtin_expect((uint32_t)(eb - 1) < 254u, 1)) return u2f(sign | ((uint32_t)eb << 23) | frac);
+    if (eb > (1 << 19)) return u2f(kQNaN);           // an inf/NaN operand
+    return u2f(join_mag(sign, eb - 127, frac));      // overflow, gradual underflow, zero
+}
+
+// Quotient of decomposed operands (a carries bias 127, b bias 0).
+__device__ __forceinline__ float pad_from_split(const Split& a, const Split& b)
+{
+    uint32_t f = a.fr - b.fr;                        // bit 31: sign (xor), bit 23: fraction borrow
+    int eb = a.ex - b.ex - (int)((f >> 23) & 1u);
+    uint32_t sign = (a.fr ^ b.fr) & kSign, frac = f & kMant;
+    if (__builtin_expect((uint32_t)(eb - 1) < 254u && (uint32_t)(b.ex + 2048) < 4096u, 1))
+        return u2f(sign | ((uint32_t)eb << 23) | frac);
+    if (a.ex > (1 << 19) || b.ex > (1 << 19)) return u2f(kQNaN);          // inf/NaN anywhere
+    if (b.ex == -4096) return u2f(a.ex == -4096 ? kQNaN : (sign | kExpo));        // x / 0, 0 / 0
+    return u2f(join_mag(sign, eb - 127, frac));
+}
+
+__device__ __forceinline__ float pam_general(uint32_t ai, uint32_t bi)
+{ return pam_from_split(split_operand(ai, 127), split_operand(bi, 0)); }
 
 // PAM product a (*) b.
 __device__ __forceinline__ float pam_mul(float a, float b)
@@ -75,18 +106,8 @@ __device__ __forceinline__ float pam_mul(float a, float b)
     return pam_general(ai, bi);
 }
 
-__device__ __noinline__ float pad_general(uint32_t ai, uint32_t bi)
-{
-    uint32_t ma = ai & ~kSign, mb = bi & ~kSign;
-    if (ma >= kExpo || mb >= kExpo) return u2f(kQNaN);
-    if (mb == 0) return u2f(ma == 0 ? kQNaN : ((ai & kSign) | kExpo));
-    if (ma == 0) return u2f(bi & kSign);
-    int ea, eb; uint32_t fa, fb;
-    split_mag(ma, ea, fa); split_mag(mb, eb, fb);
-    int E = ea - eb; uint32_t M = fa - fb;
-    if (M & kSign) { E -= 1; M += 0x00800000u; }
-    return u2f(join_mag((ai ^ bi) & kSign, E, M));
-}
+__device__ __forceinline__ float pad_general(uint32_t ai, uint32_t bi)
+{ return pad_from_split(split_operand(ai, 127), split_operand(bi, 0)); }
 
 // PAM quotient a (/) b.
 __device__ __forceinline__ float pad_div(float a, float b)

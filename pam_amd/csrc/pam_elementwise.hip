@@ -110,18 +110,6 @@ __global__ __launch_bounds__(kThreads) void ew_scalar_kernel(const float* __rest
         out[i] = op(p0[i], NIN > 1 ? p1[i] : 0.f, NIN > 2 ? p2[i] : 0.f);
 }
 
-int g_cu_count = 0;
-
-int grid_cap()
-{
-    if (g_cu_count == 0) {
-        int dev = 0; hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256 * 8;
-        g_cu_count = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
-    return g_cu_count * 8;      // eight work-groups of four wavefronts per compute unit
-}
-
 template <class Op, int NIN>
 int launch(const char* what, const float* p0, const float* p1, const float* p2, float* out, size_t n, Op op, void* stream)
 {
@@ -130,17 +118,17 @@ int launch(const char* what, const float* p0, const float* p1, const float* p2, 
     hipStream_t st = (hipStream_t)stream;
     uintptr_t align = (uintptr_t)p0 | (uintptr_t)out | (NIN > 1 ? (uintptr_t)p1 : 0) | (NIN > 2 ? (uintptr_t)p2 : 0);
     size_t nvec = (align & 15u) ? 0 : n / 4;
-    const int cap = grid_cap();
+    const size_t cap = (size_t)1 << 30;      // one pass per lane for any realistic size; grid-stride beyond
     if (nvec) {
         size_t blocks = (nvec + kThreads * kUnroll - 1) / (kThreads * kUnroll);
-        if (blocks > (size_t)cap) blocks = cap;
+        if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL((ew_vec_kernel<Op, NIN>), dim3((unsigned)blocks), dim3(kThreads), 0, st,
                            (const v4f*)p0, (const v4f*)p1, (const v4f*)p2, (v4f*)out, nvec, op);
     }
     if (nvec * 4 < n) {
         size_t rest = n - nvec * 4;
         size_t blocks = (rest + kThreads - 1) / kThreads;
-        if (blocks > (size_t)cap) blocks = cap;
+        if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL((ew_scalar_kernel<Op, NIN>), dim3((unsigned)blocks), dim3(kThreads), 0, st,
                            p0, p1, p2, out, nvec * 4, n, op);
     }

@@ -165,37 +165,6 @@ struct TileLoader {
     }
 };
 
-// Guarded PAM product on decomposed operands.  An operand is split once per k-step into
-//   ex = unbiased exponent (+127 folded into the L side), or a sentinel: -2^12 for zero,
-//        +2^20 for inf/NaN;
-//   fr = 23-bit fraction with subnormals normalised, the sign in bit 31 (cleared for zeros,
-//        whose sign the reference's float emulation ignores, pam/native.py:54).
-// A pair then costs two adds and a range check; zeros fall out of the underflow branch with
-// the sign of the other operand, inf/NaN out of the overflow branch.
-struct Split { int ex; uint32_t fr; };
-
-__device__ __forceinline__ Split split_operand(uint32_t u, int bias)
-{
-    uint32_t mag = u & ~kSign;
-    Split s;
-    if (__builtin_expect(mag - 0x00800000u < 0x7f000000u, 1)) {
-        s.ex = (int)(mag >> 23) - 127 + bias; s.fr = u & (kSign | kMant);
-    } else if (mag == 0) { s.ex = -4096; s.fr = 0; }
-    else if (mag >= kExpo) { s.ex = 1 << 20; s.fr = 0; }
-    else { int e; uint32_t m; split_mag(mag, e, m); s.ex = e + bias; s.fr = (u & kSign) | m; }
-    return s;
-}
-
-__device__ __forceinline__ float guarded_product(const Split& a, const Split& b)
-{
-    uint32_t f = a.fr + b.fr;                        // bit 31: sign, bit 23: fraction carry
-    int eb = a.ex + b.ex + (int)((f >> 23) & 1u);    // biased exponent of the product
-    uint32_t sign = f & kSign, frac = f & kMant;
-    if (__builtin_expect((uint32_t)(eb - 1) < 254u, 1)) return u2f(sign | ((uint32_t)eb << 23) | frac);
-    if (eb > (1 << 19)) return u2f(kQNaN);           // an inf/NaN operand
-    return u2f(join_mag(sign, eb - 127, frac));      // overflow, gradual underflow, zero
-}
-
 // Exact-backward product from the normalised mantissa fraction of the forward operand
 // whose gradient is wanted, the other forward operand b (offset already applied) and the
 // upstream gradient (pam/cuda_kernels.cu:48-57, pam/native.py:74-77), all classes.
@@ -347,7 +316,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] += guarded_product(sa[i], sb[j]);
+                    for (int j = 0; j < TN; ++j) acc[i][j] += pam_from_split(sa[i], sb[j]);
                 return;
             }
 #pragma unroll
