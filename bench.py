@@ -8,7 +8,7 @@ dX and dW (the approximate backward of the reference's training recipe,
 pam/cuda_bindings.py:154-161).  `value` is G PAM-MAC/s over whole steps with all operands
 resident in HBM.  Each product is also timed on its own with HIP events, which gives the
 roofline figure of the matrix kernel (VALU issue rate: 2 lane-ops per MAC against
-CUs x 64 lanes x clock), and the elementwise multiply / divide are timed on 2^26
+CUs x 128 lanes x clock), and the elementwise multiply / divide are timed on 2^26
 elements against HBM bandwidth.  The CPU baseline is this repository's own C restatement
 of the same arithmetic (oracle/, OpenMP) on the host cores, on the 192->768 layer.
 """
@@ -49,7 +49,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
-                 "(the path has no collective; see DESIGN.md for how it would shard)")
+                 "(the path has no collective: it shards by rows, with one all-reduce of dW per layer)")
     import torch
     from pam_amd import _abi
     from pam_amd._abi import HipKernels
