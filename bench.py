@@ -127,7 +127,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "DeiT-tiny PAM linear fwd+dX+dW, tokens 64x197=12608, 192->768 and 768->192 "
-                               "(BASELINE configs[2]); 6 products of 1 859 125 248 PAM-MAC per step"},
+                               "(benchmark configuration 2); 6 products of 1 859 125 248 PAM-MAC per step"},
         "roofline": roofline, "products": per,
     }
 
@@ -143,7 +143,7 @@ def main():
             ms = event_time_ms(fn, 20, torch)
             ew[name] = {"ms": round(ms, 4), "GBps": round(12 * n / ms / 1e6, 1)}
         out["roofline_elementwise"] = {
-            "kernel": "ew_vec_kernel (PAM multiply, 2^26 elements, BASELINE configs[1])", "bound": "hbm",
+            "kernel": "ew_vec_kernel (PAM multiply, 2^26 elements, benchmark configuration 1)", "bound": "hbm",
             "achieved": ew["mul"]["GBps"], "peak": 8000.0, "unit": "GB/s", "frac": round(ew["mul"]["GBps"] / 8000.0, 4),
             "traffic": traffic.get("ew_mul_2p26_bytes"), "bytes_per_element": 12, "div_GBps": ew["div"]["GBps"],
         }

@@ -25,9 +25,10 @@
 //  * While staging, every element's exponent is folded into a running min/max.  If all of a
 //    k-tile's L and R values are normal numbers with magnitude in [2^-63, 2^64), no product
 //    in the tile can leave the normal range and the two-instruction loop is exact;
-//    otherwise (zeros, subnormals, inf, NaN, extreme exponents) the work-group takes a
-//    guarded loop for that k-tile, which evaluates the full definition per product on
-//    operands decomposed once per k-step.  The choice is uniform per work-group and k-tile.
+//    a k-tile that only adds zeros to that (ReLU activations, padding) takes a loop with one
+//    extra select per product; anything else (subnormals, inf, NaN, extreme exponents) takes a
+//    guarded loop that evaluates the full definition per product on operands decomposed once
+//    per k-step.  The choice is uniform per work-group and k-tile.
 //  * Rows beyond M / N are clamped to the last valid row when loading (their results are
 //    never stored); the k tail runs a shorter loop, padding never enters the arithmetic.
 //  * Shapes with few output tiles and long k (dX: 12608 x 192, k = 768; dW: 192 x 768,
@@ -59,15 +60,19 @@ struct GemmArgs {
     float off; int has_off;
 };
 
-// Classifies and transforms one staged value.  MODE_PAM: R carries the bias subtraction.
+// Classifies and transforms one staged value.  MODE_PAM: R carries the bias subtraction, and
+// zeros are staged in one canonical pattern (their sign never shows in a sum that starts at +0).
 // Backward modes: the "slope side" is the forward operand b of pam_bwd(a, b, delta).
+constexpr uint32_t kZeroL = 0u;                 // canonical staged zero of L
+constexpr uint32_t kZeroR = 0u - kBias;         // canonical staged zero of R (bias already subtracted)
+
 template <int MODE, bool IS_R>
 struct Stager {
     static constexpr bool kSlopeSide = (MODE == MODE_BWD_DL && IS_R) || (MODE == MODE_BWD_DR && !IS_R);
     static constexpr bool kDeltaSide = (MODE >= MODE_BWD_DL) && !kSlopeSide;
     static constexpr bool kTakesOffset = (MODE == MODE_PAM && IS_R) || kSlopeSide;
     uint32_t emin = 255u, emax = 0u;
-    bool bad = false;
+    bool bad = false, zero = false;
 
     __device__ __forceinline__ uint32_t one(float v)
     {
@@ -78,11 +83,20 @@ struct Stager {
             return u;
         }
         uint32_t e = (u >> 23) & 0xffu;
+        if (MODE == MODE_PAM) {                    // zeros get their own, cheaper loop
+            bool z = (u & ~kSign) == 0;
+            zero |= z;
+            e = z ? 127u : e;
+            emin = min(emin, e); emax = max(emax, e);
+            return z ? (IS_R ? kZeroR : kZeroL) : (IS_R ? u - kBias : u);
+        }
         emin = min(emin, e); emax = max(emax, e);
-        return (MODE == MODE_PAM && IS_R) ? u - kBias : u;
+        return u;
     }
-    // true when some staged value lies outside [2^-63, 2^64) or is not a normal number
-    __device__ __forceinline__ bool guarded() const { return bad || emin < 64u || emax > 190u; }
+    // 2: some staged value lies outside [2^-63, 2^64) or is not a normal number or zero;
+    // 1: all non-zero values are inside, but there are zeros; 0: the plain loop is exact
+    __device__ __forceinline__ uint32_t verdict() const
+    { return (bad || emin < 64u || emax > 190u) ? 2u : zero ? 1u : 0u; }
 };
 
 // One operand's tile: ROWS x BK values from global memory into registers, then into LDS.
@@ -249,8 +263,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
         ll.store(lds_l[buf], tid, sl);
         rl.store(lds_r[buf], tid, sr);
         if (MODE != MODE_STD) {
-            unsigned long long any = __ballot(sl.guarded() || sr.guarded());
-            if (lane == 0) lds_flag[buf][wave] = any != 0ull;
+            uint32_t v = max(sl.verdict(), sr.verdict());
+            uint32_t worst = __ballot(v == 2u) != 0ull ? 2u : __ballot(v == 1u) != 0ull ? 1u : 0u;
+            if (lane == 0) lds_flag[buf][wave] = worst;
         }
     };
 
@@ -269,12 +284,12 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
             rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid);
         }
         const int kcount = min(BK, kend - k0);
-        bool guarded = false;
+        uint32_t verdict = 0;                     // 0 plain loop, 1 zeros present, 2 guarded
         if (MODE != MODE_STD) {
             uint32_t f = 0;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) f |= lds_flag[cur][w];
-            guarded = __builtin_amdgcn_readfirstlane(f) != 0;
+            for (int w = 0; w < NW; ++w) f = max(f, lds_flag[cur][w]);
+            verdict = __builtin_amdgcn_readfirstlane(f);
         }
         const uint32_t* sl = lds_l[cur] + ty * 4;
         const uint32_t* sr = lds_r[cur] + tx * 4;
@@ -304,6 +319,21 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
                     else acc[i][j] = fmaf(u2f(b[j]), u2f((a[i] + dfrac[i][j]) & ~kMant), acc[i][j]);
                 }
         };
+        // k-tile with zeros but otherwise in range: the integer add of a zero is garbage, so those
+        // products are replaced by +0 (one v_cndmask per product, masks combined on the scalar unit)
+        auto zeros_step = [&](int kk) {
+            uint32_t a[TM], b[TN];
+            fragment(kk, a, b);
+            bool za[TM], zb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) za[i] = a[i] == kZeroL;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) zb[j] = b[j] == kZeroR;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] += u2f((za[i] | zb[j]) ? 0u : a[i] + b[j]);
+        };
         auto guarded_step = [&](int kk) {
             uint32_t a[TM], b[TN];
             fragment(kk, a, b);
@@ -328,7 +358,10 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
                 }
         };
 
-        if (!guarded) {
+        if (verdict == 1 && MODE == MODE_PAM) {
+#pragma unroll 2
+            for (int kk = 0; kk < kcount; ++kk) zeros_step(kk);
+        } else if (verdict == 0) {
             if (kcount == BK) {
 #pragma unroll 4
                 for (int kk = 0; kk < BK; ++kk) fast_step(kk);

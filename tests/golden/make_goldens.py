@@ -146,7 +146,7 @@ def main():
         d[f"{tag}_da_approx"] = u32(A2.grad); d[f"{tag}_db_approx"] = u32(B2.grad.contiguous())
     np.savez_compressed(OUT / "matmul_small.npz", **d)
 
-    # ---- 7. BASELINE config 0: A[256,512] @ B[512,256], seeds 0/1/2, fwd + approx bwd
+    # ---- 7. benchmark configuration 0: A[256,512] @ B[512,256], seeds 0/1/2, fwd + approx bwd
     A = torch.randn(256, 512, generator=torch.Generator().manual_seed(0)).requires_grad_()
     B = torch.randn(512, 256, generator=torch.Generator().manual_seed(1)).requires_grad_()
     dY = torch.randn(256, 256, generator=torch.Generator().manual_seed(2))
