@@ -313,6 +313,40 @@ def test_deit_linear_full_size(K, oracle):
     assert torch.equal(K.pam_matmul_fwd(tX[perm], tW.T, True, False, 1.0), Y[perm])
 
 
+def test_attention_bmm_full_size(K, oracle):
+    """Batched attention products at full size (batch 64 x 3 heads, 197 tokens, head dim 64): Q K^T and
+    P V forward plus the approximate backward products on transposed views, sampled batches
+    against the oracle; K = 197 (prime) and 64 exercise the k tail and the row tails."""
+    g = torch.Generator().manual_seed(300)
+    B, T, D = 192, 197, 64
+    Q, Kk, V = (torch.randn(B, T, D, generator=g) for _ in range(3))
+    P = torch.softmax(torch.randn(B, T, T, generator=g), dim=-1)
+    dS, dO = torch.randn(B, T, T, generator=g), torch.randn(B, T, D, generator=g)
+    q, k, v, p, ds, do = (t.cuda() for t in (Q, Kk, V, P, dS, dO))
+    kt = k.transpose(1, 2)
+    S = K.pam_bmm_fwd(q, kt, True, False, 1.0)                   # [B, T, T], K = 64
+    O = K.pam_bmm_fwd(p, v, True, True, 1.0)                     # [B, T, D], K = 197
+    dQ = K.pam_bmm_fwd(ds, kt.mT, True, True, 1.0)               # dS K
+    dKt = K.pam_bmm_fwd(q.mT, ds, False, True, 1.0)              # Q^T dS
+    dP = K.pam_bmm_fwd(do, v.mT, True, False, 1.0)               # dO V^T
+    dV = K.pam_bmm_fwd(p.mT, do, False, True, 1.0)               # P^T dO
+    pick = [0, 77, 191]
+    n = lambda t: t[pick].numpy()
+    tr = lambda a: np.swapaxes(a, 1, 2)
+    cases = [("S", S, n(Q), tr(n(Kk)), (B, T, T, D)), ("O", O, n(P), n(V), (B, T, D, T)),
+             ("dQ", dQ, n(dS), n(Kk), (B, T, D, T)), ("dKt", dKt, tr(n(Q)), n(dS), (B, D, T, T)),
+             ("dP", dP, n(dO), tr(n(V)), (B, T, T, D)), ("dV", dV, tr(n(P)), n(dO), (B, T, D, T))]
+    for name, got, L, R, shape in cases:
+        assert_same_bits(host(got)[pick], ogemm(oracle, L, R, plan_shape=shape), name)
+    # the autograd layer produces the same six tensors
+    import pam_amd as pam
+    q2, k2, v2, p2 = (t.clone().requires_grad_() for t in (q, k, v, p))
+    s2 = pam.bmm(q2, k2.transpose(1, 2), approx_bwd=True); s2.backward(ds)
+    o2 = pam.bmm(p2, v2, approx_bwd=True); o2.backward(do)
+    assert torch.equal(s2, S) and torch.equal(o2, O) and torch.equal(q2.grad, dQ) and torch.equal(p2.grad, dP)
+    assert torch.equal(k2.grad, dKt.transpose(1, 2)) and torch.equal(v2.grad, dV)
+
+
 def test_elementwise_full_size(K, oracle):
     """2^26 elements, 98 % N(0,1) and 2 % edge values: slices against the oracle, and the
     round trip (a (*) b) (/) b == a wherever nothing saturates."""
