@@ -7,5 +7,7 @@ The names of the reference's `pam` package that live on this path are re-exporte
 (pam/__init__.py:8-10).
 """
 from .pam_ops import *          # noqa: F401,F403
+from .composites import *       # noqa: F401,F403
 from . import cuda_bindings     # noqa: F401
 from . import pam_ops           # noqa: F401
+from . import composites        # noqa: F401

@@ -60,7 +60,7 @@ class OracleKernels:
         return t.detach().numpy()
 
     def _ret(self, a):
-        return torch.from_numpy(np.ascontiguousarray(a))
+        return torch.from_numpy(np.array(a, dtype=np.float32, order="C"))      # keeps 0-d results 0-d
 
     def _off(self, offset):
         return None if offset == 1.0 else offset
