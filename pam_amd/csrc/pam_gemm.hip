@@ -18,8 +18,9 @@
 //    memory, so the backward products run on the views the autograd layer hands over
 //    (pam/cuda_bindings.py:147-164).
 //  * Global loads for k-tile t+1 are issued before the arithmetic of tile t (register
-//    double buffering), LDS is double buffered, one barrier per k-tile.  k-tiles are 32
-//    deep for long k and 16 deep for short k.
+//    double buffering), LDS is double buffered, one barrier per k-tile, and inside a k-tile
+//    the fragments of step k+1 are read while step k is computed.  k-tiles are 32 deep for
+//    long k and 16 deep for short k.
 //  * The bias subtraction and the optional offset (R' = R (*) offset) are applied once per
 //    element while staging R.
 //  * While staging, every element's exponent is folded into a running min/max.  If all of a
@@ -363,8 +364,22 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
             for (int kk = 0; kk < kcount; ++kk) zeros_step(kk);
         } else if (verdict == 0) {
             if (kcount == BK) {
-#pragma unroll 4
-                for (int kk = 0; kk < BK; ++kk) fast_step(kk);
+                // fragments for step kk+1 are read from LDS while step kk is computed
+                uint32_t fa[2][TM], fb[2][TN];
+                fragment(0, fa[0], fb[0]);
+#pragma unroll
+                for (int kk = 0; kk < BK; ++kk) {
+                    if (kk + 1 < BK) fragment(kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j) {
+                            if (MODE == MODE_PAM) acc[i][j] += u2f(fa[kk & 1][i] + fb[kk & 1][j]);
+                            else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f(fb[kk & 1][j]), acc[i][j]);
+                            else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f((fb[kk & 1][j] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                            else acc[i][j] = fmaf(u2f(fb[kk & 1][j]), u2f((fa[kk & 1][i] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                        }
+                }
             } else {
 #pragma unroll 1
                 for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
