@@ -14,6 +14,7 @@ of the same arithmetic (oracle/, OpenMP) on the host cores, on the 192->768 laye
 """
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -150,7 +151,36 @@ def main():
         if args.copy_probe:
             c = torch.empty_like(a)
             c.copy_(b); torch.cuda.synchronize()
-        del a, b
+            del c
+        # the other kernels of the path, each against its own bound (not part of `value`)
+        d = torch.randn(n, generator=g).to(dev)
+        other = {}
+        stream_ops = (
+            ("pam_bwd", 16, lambda: K.pam_bwd(a, b, d, 1.0)), ("pad_bwd", 16, lambda: K.pad_bwd(a, b, d, 1.0)),
+            ("pam_fwd_offset", 12, lambda: K.pam_fwd(a, b, 1.0552)),
+            ("pam_fwd_scalar_operand", 8, lambda: K.pam_fwd(a, d[:1].expand(n), 1.0)),
+            ("pa_exp_fwd", 8, lambda: K.pa_exp_fwd(d, math.e, 1.0)), ("pa_log_fwd", 8, lambda: K.pa_log_fwd(a, math.e, 1.0)),
+            ("pa_exp_bwd", 12, lambda: K.pa_exp_bwd(d, b, math.e, 1.0)), ("pa_log_bwd", 12, lambda: K.pa_log_bwd(a, b, math.e, 1.0)),
+        )
+        for name, bpe, fn in stream_ops:
+            ms = event_time_ms(fn, 10, torch)
+            other[name] = {"ms": round(ms, 4), "GBps": round(bpe * n / ms / 1e6, 1), "hbm_frac": round(bpe * n / ms / 1e6 / 8000.0, 3)}
+        del a, b, d
+        # exact backward products (3 lane-ops per MAC) and the attention products of configuration 3
+        Xd = X1.contiguous()
+        exact = {
+            "exact_dX_12608x192x768": (3, macs_each, lambda: K.pam_matmul_bwd(dY1, W1, Xd, True, True, True, 1.0)),
+            "exact_dW_192x768x12608": (3, macs_each, lambda: K.pam_matmul_bwd(X1.T, dY1, W1.T, False, True, False, 1.0)),
+        }
+        Bh, Tk, Dh = 192, 197, 64
+        q, kk, v = (torch.randn(Bh, Tk, Dh, generator=g).to(dev) for _ in range(3))
+        pr = torch.softmax(torch.randn(Bh, Tk, Tk, generator=g), -1).to(dev)
+        exact["bmm_QKt_192x197x197x64"] = (2, Bh * Tk * Tk * Dh, lambda: K.pam_bmm_fwd(q, kk.transpose(1, 2), True, False, 1.0))
+        exact["bmm_PV_192x197x64x197"] = (2, Bh * Tk * Tk * Dh, lambda: K.pam_bmm_fwd(pr, v, True, True, 1.0))
+        for name, (ops, macs, fn) in exact.items():
+            ms = event_time_ms(fn, 10, torch)
+            other[name] = {"ms": round(ms, 4), "gmacs": round(macs / ms / 1e6, 1), "valu_frac": round(ops * macs / (ms * 1e-3) / lane_peak, 4)}
+        out["other_kernels"] = other
 
     if not args.no_cpu_baseline:
         from oracle import pam_oracle as oracle
