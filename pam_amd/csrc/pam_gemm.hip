@@ -144,9 +144,12 @@ struct TileLoader {
     // R' = R (*) offset, once per element (uniform branch around the whole tile)
     __device__ __forceinline__ void apply_offset(float off)
     {
-        float* s = reinterpret_cast<float*>(v);
-#pragma unroll 1
-        for (int i = 0; i < kElems; ++i) s[i] = pam_mul(s[i], off);
+        // fully unrolled: a run-time index would push the register tile into scratch memory
+#pragma unroll
+        for (int i = 0; i < (kVecs > 0 ? kVecs : 1); ++i) {
+            v[i].x = pam_mul(v[i].x, off); v[i].y = pam_mul(v[i].y, off);
+            v[i].z = pam_mul(v[i].z, off); v[i].w = pam_mul(v[i].w, off);
+        }
     }
 
     template <class S>
