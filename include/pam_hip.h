@@ -2,7 +2,7 @@
  * pam_hip.h -- C ABI of libpam_hip.so, the MI355X (gfx950) implementation of the
  * piecewise-affine arithmetic kernels of epfml/pam.
  *
- * The fourteen compute entry points are the fourteen functions of the reference's
+ * The fourteen primitive entry points are the fourteen functions of the reference's
  * extension module (PYBIND11_MODULE in pam/cuda_kernels.cu:932-947), one to one and under
  * the same names with a pam_hip_ prefix.  Where the reference takes torch tensors and
  * returns a new one, these take raw device pointers plus sizes and element strides and
@@ -113,6 +113,37 @@ int pam_hip_pam_matmul_bwd(const float *l, long l_sr, long l_sc, const float *r,
 int pam_hip_pam_bmm_bwd(PAM_HIP_MAT(l), PAM_HIP_MAT(r), PAM_HIP_MAT(mo), PAM_HIP_OUT(dm),
                         long batch, long m, long n, long k, int delta_l, float offset,
                         void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- row-wise compositions as single kernels (pam/pam_ops.py:288-378) ------------------- */
+/* The reference builds these from five to fifteen elementwise launches; the entry points
+ * below compute, element for element, the same chain of primitive calls in one sweep over
+ * x[rows][n] (contiguous rows, the reduced dimension last).  The order of each row sum,
+ * which the reference leaves to torch.sum, is fixed: lane l of 64 adds the elements
+ * l, l + 64, ... in ascending order from +0, then p[l] = p[l] + p[l ^ s] for
+ * s = 32, 16, 8, 4, 2, 1. */
+/* Bytes of device scratch the softmax / logsumexp entry points need (block maxima). */
+size_t pam_hip_rowop_workspace_bytes(void);
+/* y = softmax(x) over the last dim        replaces pam.softmax (pam/pam_ops.py:305-328):
+ * x (*) log2 e with -inf kept, one global shift floor(max) written to shift[0], exp2, row
+ * sum written to row_sum[rows], (/) by it. */
+int pam_hip_softmax_fwd(const float *x, float *y, float *row_sum, float *shift, long rows, long n, float offset,
+                        void *workspace, size_t workspace_bytes, void *stream);
+/* dx for the above from the upstream gradient dy, following the autograd chain of the
+ * primitives (pam/cuda_bindings.py:43-57, 78-97, 224-239).  approx_a / approx_b select the
+ * approximate gradient for first / second operands of the products and quotients,
+ * approx_exp the one of exp2; row_sum and shift are the forward's outputs. */
+int pam_hip_softmax_bwd(const float *x, const float *dy, const float *row_sum, const float *shift, float *dx,
+                        long rows, long n, float offset, int approx_a, int approx_b, int approx_exp, void *stream);
+/* lse[rows] = logsumexp(x) over the last dim and/or log_softmax[rows][n] = x - lse (either
+ * pointer may be NULL)                    replaces pam.logsumexp / pam.log_softmax (:331-347) */
+int pam_hip_logsumexp_fwd(const float *x, float *lse, float *log_softmax, long rows, long n, float offset,
+                          void *workspace, size_t workspace_bytes, void *stream);
+/* y[rows] = sum(x[row]) (/) n             replaces pam.mean over the last dim (:288-302) */
+int pam_hip_row_mean_fwd(const float *x, float *y, long rows, long n, float offset, void *stream);
+/* y = layer_norm(x) over the last dim, weight and bias of n elements or NULL
+ *                                          replaces pam.layer_norm (:350-378) */
+int pam_hip_layer_norm_fwd(const float *x, const float *weight, const float *bias, float *y, long rows, long n,
+                           float eps, float offset, void *stream);
 
 #ifdef __cplusplus
 }

@@ -36,6 +36,12 @@
  *                                      pam/cuda_kernels.cu:85-136,375-393,470-486:
  *                                      the reference has no CPU implementation and
  *                                      no test of them.
+ *   row-wise compositions ............ equal, bit for bit, to the same chain built from
+ *                                      the pinned primitives above whenever the row sums
+ *                                      are exact (short-mantissa rows), and to it within
+ *                                      summation-order noise otherwise; the softmax
+ *                                      gradient likewise against the primitives' backward
+ *                                      formulas chained by hand (tests/test_rowops.py)
  *   GEMM ............................. power-of-two operands == fp32 matmul
  *                                      (pam/test_pam.py:151-216 construction), the
  *                                      reference's deterministic 5x4 / 4x3 operands
@@ -44,6 +50,7 @@
 #include <math.h>
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include <string.h>
 
 #define BIAS_BITS 0x3f800000u
@@ -401,4 +408,147 @@ void pamo_gemm_fast(long M, long N, long K, const float *L, const float *R, floa
     }
 }
 
-int pamo_version(void) { return 1; }
+/* ------------------------------------------------------------------ row-wise compositions
+ * softmax, logsumexp / log_softmax, mean and layer_norm of the reference's op library
+ * (pam/pam_ops.py:288-378) written out as the chain of primitive calls they make, and the
+ * softmax gradient as autograd chains the primitives' backward formulas
+ * (pam/cuda_bindings.py:43-57, 78-97, 224-239).  The one thing the reference leaves open,
+ * the order of torch.sum along a row, is fixed to the order of the GPU kernels:
+ * 64 strided partial sums from +0, then a butterfly p[l] = p[l] + p[l ^ s], s = 32 .. 1. */
+static float row_sum_fixed(const float *v, long n)
+{
+    float p[64], q[64];
+    for (int l = 0; l < 64; ++l) {
+        volatile float s = 0.0f;
+        for (long i = l; i < n; i += 64) s = s + v[i];
+        p[l] = s;
+    }
+    for (int s = 32; s >= 1; s >>= 1) {
+        for (int l = 0; l < 64; ++l) { volatile float t = p[l] + p[l ^ s]; q[l] = t; }
+        memcpy(p, q, sizeof p);
+    }
+    return p[0];
+}
+
+static float *row_buffer(long n) { return (float *)malloc(sizeof(float) * (size_t)(n > 0 ? n : 1)); }
+
+static const float LOG2_E = (float)1.4426950408889634;   /* math.log2(math.e) as an fp32 tensor */
+static const float LN_2 = (float)0.6931471805599453;     /* math.log(2.0) as an fp32 tensor */
+
+static int is_neg_inf(float x) { return f2u(x) == 0xff800000u; }
+static float scaled_x(float x, float off, int mask_inf)
+{ return (mask_inf && is_neg_inf(x)) ? x : pam_off(x, LOG2_E, off); }
+static float exp2_op(float t, float off) { return paexp(t, 1.0f, off); }     /* pa_exp_fwd(base 2) */
+static float log2_op(float v, float off) { return palog(v, 1.0f, off); }     /* pa_log_fwd(base 2) */
+
+/* floor(max) over the whole tensor, NaN propagating like torch.max (pam/pam_ops.py:318-319) */
+static float global_shift(const float *x, size_t count, float off, int mask_inf)
+{
+    float mx = -INFINITY; int nan = 0;
+    for (size_t i = 0; i < count; ++i) {
+        float v = scaled_x(x[i], off, mask_inf);
+        if (isnan(v)) nan = 1; else if (v > mx) mx = v;
+    }
+    return nan ? NAN : floorf(mx);
+}
+
+static float softmax_weight(float x, float shift, float off)
+{
+    if (is_neg_inf(x)) return 0.0f;
+    volatile float t = scaled_x(x, off, 0) - shift;
+    return exp2_op(t, off);
+}
+
+void pamo_softmax_fwd(const float *x, float *y, float *row_sum, float *shift_out, long rows, long n, float off)
+{
+    float shift = global_shift(x, (size_t)rows * (size_t)n, off, 1);
+    *shift_out = shift;
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) {
+        float *e = row_buffer(n);
+        for (long i = 0; i < n; ++i) e[i] = softmax_weight(x[r * n + i], shift, off);
+        float total = row_sum_fixed(e, n);
+        for (long i = 0; i < n; ++i) y[r * n + i] = pad_off(e[i], total, off);
+        row_sum[r] = total;
+        free(e);
+    }
+}
+
+void pamo_softmax_bwd(const float *x, const float *dy, const float *row_sum, float shift, float *dx,
+                      long rows, long n, float off, int approx_a, int approx_b, int approx_exp)
+{
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) {
+        const float *xr = x + r * n, *g = dy + r * n;
+        float total = row_sum[r], inv = pad_off(1.0f, total, off);
+        float *e = row_buffer(n), *term = row_buffer(n);
+        for (long i = 0; i < n; ++i) {
+            e[i] = softmax_weight(xr[i], shift, off);
+            /* pad_autograd.backward, second operand (the broadcast row sum) */
+            if (approx_b) { volatile float t = pam_off(pad_off(pad_off(e[i], total, off), total, off), g[i], off); term[i] = -t; }
+            else term[i] = pad_bwd1(e[i], total, g[i], off);
+        }
+        float dtotal = row_sum_fixed(term, n);          /* gradient of the expanded row sum */
+        for (long i = 0; i < n; ++i) {
+            int masked = is_neg_inf(xr[i]);
+            float de0 = approx_a ? pam_off(inv, g[i], off) : pam_bwd1(e[i], inv, g[i], 1.0f);
+            volatile float de = de0 + dtotal;            /* pad's first operand + the sum's broadcast */
+            if (masked) de = 0.0f;                       /* where(x == -inf, 0, exp2(..)) */
+            volatile float t = scaled_x(xr[i], off, 1) - shift;
+            float dt;
+            if (approx_exp) dt = pam_off(pam_off(exp2_op(t, off), LN_2, off), de, off);
+            else dt = paexp_bwd(t, de, 1.0f, off);
+            if (masked) dt = 0.0f;                       /* where(x == -inf, -inf, mul(..)) */
+            dx[r * n + i] = approx_a ? pam_off(dt, LOG2_E, off) : pam_bwd1(xr[i], LOG2_E, dt, off);
+        }
+        free(e); free(term);
+    }
+}
+
+/* lse[r] and/or y[r][i] = x - lse (either may be NULL) */
+void pamo_logsumexp_fwd(const float *x, float *lse, float *y, long rows, long n, float off)
+{
+    float shift = global_shift(x, (size_t)rows * (size_t)n, off, 0);
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) {
+        float *e = row_buffer(n);
+        for (long i = 0; i < n; ++i) { volatile float t = scaled_x(x[r * n + i], off, 0) - shift; e[i] = exp2_op(t, off); }
+        float total = row_sum_fixed(e, n);
+        free(e);
+        volatile float s = shift + log2_op(total, off);
+        float out = pad_off(s, LOG2_E, off);
+        if (lse) lse[r] = out;
+        if (y) for (long i = 0; i < n; ++i) { volatile float d = x[r * n + i] - out; y[r * n + i] = d; }
+    }
+}
+
+void pamo_row_mean_fwd(const float *x, float *y, long rows, long n, float off)
+{
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) y[r] = pad_off(row_sum_fixed(x + r * n, n), (float)n, off);
+}
+
+void pamo_layer_norm_fwd(const float *x, const float *weight, const float *bias, float *y, long rows, long n,
+                         float eps, float off)
+{
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) {
+        const float *xr = x + r * n;
+        float *c = row_buffer(n), *q = row_buffer(n);
+        float mu = pad_off(row_sum_fixed(xr, n), (float)n, off);
+        for (long i = 0; i < n; ++i) { volatile float d = xr[i] - mu; c[i] = d; q[i] = pam_off(d, d, off); }
+        float var = pad_off(row_sum_fixed(q, n), (float)n, off);
+        volatile float v = var + eps;
+        /* pow(v, 0.5) (pam/pam_ops.py:70-79) */
+        float denom = v == 0.0f ? 0.0f : exp2_op(pam_off(log2_op(v, off), 0.5f, off), off);
+        for (long i = 0; i < n; ++i) {
+            float out = pad_off(c[i], denom, off);
+            if (weight) out = pam_off(out, weight[i], off);
+            if (bias) { volatile float b = out + bias[i]; out = b; }
+            y[r * n + i] = out;
+        }
+        free(c); free(q);
+    }
+}
+
+int pamo_version(void) { return 2; }

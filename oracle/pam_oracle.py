@@ -57,6 +57,15 @@ def lib():
         L.pamo_gemm.restype = None
         L.pamo_gemm_fast.argtypes = [cl, cl, cl, _fp, _fp, _fp]
         L.pamo_gemm_fast.restype = None
+        cf, ci = ctypes.c_float, ctypes.c_int
+        L.pamo_softmax_fwd.argtypes = [_fp, _fp, _fp, _fp, cl, cl, cf]
+        L.pamo_softmax_bwd.argtypes = [_fp, _fp, _fp, cf, _fp, cl, cl, cf, ci, ci, ci]
+        L.pamo_logsumexp_fwd.argtypes = [_fp, _fp, _fp, cl, cl, cf]
+        L.pamo_row_mean_fwd.argtypes = [_fp, _fp, cl, cl, cf]
+        L.pamo_layer_norm_fwd.argtypes = [_fp, _fp, _fp, _fp, cl, cl, cf, cf]
+        for name in ("pamo_softmax_fwd", "pamo_softmax_bwd", "pamo_logsumexp_fwd", "pamo_row_mean_fwd",
+                     "pamo_layer_norm_fwd"):
+            getattr(L, name).restype = None
     return _lib
 
 
@@ -199,3 +208,53 @@ def gemm_fast(L, R):
     Y = np.empty((M, N), dtype=np.float32)
     lib().pamo_gemm_fast(M, N, K, _p(L), _p(R), _p(Y))
     return Y
+
+
+# ---- row-wise compositions over the last dimension (fixed summation order) ----
+
+def _rows(x):
+    x = _f32(x)
+    n = x.shape[-1]
+    return x.reshape(-1, n), x.shape
+
+
+def softmax_fwd(x, offset=None):
+    """Returns (y, row_sum[rows], shift)."""
+    x2, shape = _rows(x)
+    y = np.empty_like(x2); rs = np.empty(x2.shape[0], dtype=np.float32); shift = np.empty(1, dtype=np.float32)
+    lib().pamo_softmax_fwd(_p(x2), _p(y), _p(rs), _p(shift), x2.shape[0], x2.shape[1], _off(offset))
+    return y.reshape(shape), rs, shift[0]
+
+
+def softmax_bwd(x, dy, row_sum, shift, offset=None, approx=(False, False, False)):
+    x2, shape = _rows(x); dy2, _ = _rows(dy)
+    rs = _f32(row_sum); dx = np.empty_like(x2)
+    lib().pamo_softmax_bwd(_p(x2), _p(dy2), _p(rs), float(shift), _p(dx), x2.shape[0], x2.shape[1], _off(offset),
+                           int(approx[0]), int(approx[1]), int(approx[2]))
+    return dx.reshape(shape)
+
+
+def logsumexp_fwd(x, offset=None, with_log_softmax=False):
+    x2, shape = _rows(x)
+    lse = np.empty(x2.shape[0], dtype=np.float32)
+    y = np.empty_like(x2) if with_log_softmax else None
+    lib().pamo_logsumexp_fwd(_p(x2), _p(lse), _p(y) if with_log_softmax else None, x2.shape[0], x2.shape[1], _off(offset))
+    lse = lse.reshape(shape[:-1])
+    return (lse, y.reshape(shape)) if with_log_softmax else lse
+
+
+def row_mean_fwd(x, offset=None):
+    x2, shape = _rows(x)
+    y = np.empty(x2.shape[0], dtype=np.float32)
+    lib().pamo_row_mean_fwd(_p(x2), _p(y), x2.shape[0], x2.shape[1], _off(offset))
+    return y.reshape(shape[:-1])
+
+
+def layer_norm_fwd(x, weight=None, bias=None, eps=1e-5, offset=None):
+    x2, shape = _rows(x)
+    w = None if weight is None else _f32(weight).ravel()
+    b = None if bias is None else _f32(bias).ravel()
+    y = np.empty_like(x2)
+    lib().pamo_layer_norm_fwd(_p(x2), None if w is None else _p(w), None if b is None else _p(b), _p(y),
+                              x2.shape[0], x2.shape[1], float(np.float32(eps)), _off(offset))
+    return y.reshape(shape)

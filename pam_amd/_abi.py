@@ -43,6 +43,12 @@ _SIGNATURES = {
     "pam_hip_standard_bmm": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_matmul_bwd": (_MAT2 * 4 + [_l, _l, _l, _i, _f, _p, _z, _p], _i),
     "pam_hip_pam_bmm_bwd": (_MAT * 4 + [_l, _l, _l, _l, _i, _f, _p, _z, _p], _i),
+    "pam_hip_rowop_workspace_bytes": ([], _z),
+    "pam_hip_softmax_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_softmax_bwd": ([_p, _p, _p, _p, _p, _l, _l, _f, _i, _i, _i, _p], _i),
+    "pam_hip_logsumexp_fwd": ([_p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_row_mean_fwd": ([_p, _p, _l, _l, _f, _p], _i),
+    "pam_hip_layer_norm_fwd": ([_p, _p, _p, _p, _l, _l, _f, _f, _p], _i),
 }
 
 _lib = None
@@ -252,3 +258,79 @@ class HipKernels:
 
     def pam_bmm_bwd(self, L, R, M, L_row_major, R_row_major, delta_L, offset):
         return self._product("pam_bmm_bwd", True, L, R, M, [int(bool(delta_L))], offset)
+
+
+class HipRowKernels:
+    """Row-wise compositions over the last dimension of a contiguous [rows, n] tensor, one
+    kernel each (softmax forward and backward, logsumexp / log_softmax, row mean,
+    layer_norm); the order of their row sums is the one include/pam_hip.h states."""
+
+    @staticmethod
+    def _rows(name, X, *others):
+        _check(X, *[t for t in others if t is not None])
+        if X.dim() != 2 or not X.is_contiguous():
+            raise ValueError(f"{name}: expected a contiguous 2-D tensor")
+        for t in others:
+            if t is not None and not t.is_contiguous():
+                raise ValueError(f"{name}: operands must be contiguous")
+        return X.shape
+
+    @staticmethod
+    def _workspace(device):
+        nbytes = load_library().pam_hip_rowop_workspace_bytes()
+        return torch.empty(nbytes // 4, dtype=torch.float32, device=device), nbytes
+
+    def softmax_fwd(self, X, offset):
+        rows, n = self._rows("softmax_fwd", X)
+        Y = torch.empty_like(X)
+        row_sum = torch.empty(rows, dtype=torch.float32, device=X.device)
+        shift = torch.empty(1, dtype=torch.float32, device=X.device)
+        if X.numel():
+            with torch.cuda.device(X.device):
+                ws, nbytes = self._workspace(X.device)
+                _call("pam_hip_softmax_fwd", X.data_ptr(), Y.data_ptr(), row_sum.data_ptr(), shift.data_ptr(), rows, n,
+                      float(offset), ws.data_ptr(), nbytes, _stream())
+        return Y, row_sum, shift
+
+    def softmax_bwd(self, X, dY, row_sum, shift, offset, approx_a, approx_b, approx_exp):
+        rows, n = self._rows("softmax_bwd", X, dY, row_sum, shift)
+        if dY.shape != X.shape or row_sum.numel() != rows or shift.numel() != 1:
+            raise ValueError("softmax_bwd: operand shapes do not match")
+        dX = torch.empty_like(X)
+        if X.numel():
+            with torch.cuda.device(X.device):
+                _call("pam_hip_softmax_bwd", X.data_ptr(), dY.data_ptr(), row_sum.data_ptr(), shift.data_ptr(),
+                      dX.data_ptr(), rows, n, float(offset), int(bool(approx_a)), int(bool(approx_b)),
+                      int(bool(approx_exp)), _stream())
+        return dX
+
+    def logsumexp_fwd(self, X, offset, want_lse=True, want_log_softmax=False):
+        rows, n = self._rows("logsumexp_fwd", X)
+        lse = torch.empty(rows, dtype=torch.float32, device=X.device) if want_lse else None
+        Y = torch.empty_like(X) if want_log_softmax else None
+        if X.numel():
+            with torch.cuda.device(X.device):
+                ws, nbytes = self._workspace(X.device)
+                _call("pam_hip_logsumexp_fwd", X.data_ptr(), lse.data_ptr() if want_lse else None,
+                      Y.data_ptr() if want_log_softmax else None, rows, n, float(offset), ws.data_ptr(), nbytes, _stream())
+        return lse, Y
+
+    def row_mean_fwd(self, X, offset):
+        rows, n = self._rows("row_mean_fwd", X)
+        Y = torch.empty(rows, dtype=torch.float32, device=X.device)
+        if rows:
+            with torch.cuda.device(X.device):
+                _call("pam_hip_row_mean_fwd", X.data_ptr(), Y.data_ptr(), rows, n, float(offset), _stream())
+        return Y
+
+    def layer_norm_fwd(self, X, weight, bias, eps, offset):
+        rows, n = self._rows("layer_norm_fwd", X, weight, bias)
+        for t in (weight, bias):
+            if t is not None and t.numel() != n:
+                raise ValueError("layer_norm_fwd: weight and bias must have one value per column")
+        Y = torch.empty_like(X)
+        if X.numel():
+            with torch.cuda.device(X.device):
+                _call("pam_hip_layer_norm_fwd", X.data_ptr(), None if weight is None else weight.data_ptr(),
+                      None if bias is None else bias.data_ptr(), Y.data_ptr(), rows, n, float(eps), float(offset), _stream())
+        return Y

@@ -9,7 +9,7 @@ import subprocess
 import sys
 
 HERE = pathlib.Path(__file__).resolve().parent
-SOURCES = [HERE / "csrc" / "pam_elementwise.hip", HERE / "csrc" / "pam_gemm.hip"]
+SOURCES = [HERE / "csrc" / "pam_elementwise.hip", HERE / "csrc" / "pam_gemm.hip", HERE / "csrc" / "pam_rowops.hip"]
 LIB = HERE / "lib" / "libpam_hip.so"
 
 FLAGS = [

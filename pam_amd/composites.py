@@ -3,17 +3,31 @@ LayerNorm, conv2d, conv2d_group, Conv2d -- the rest of the reference's pam/pam_o
 (:118-257, 288-404).  Every multiply, divide, exp and log inside them is a PAM kernel call;
 additions, subtractions, maxima and sums are ordinary fp32 torch operations, as in the
 reference.  Same names and keyword arguments.
+
+Reductions over the last dimension of a contiguous GPU tensor take the single-kernel path of
+`pam_amd.fused` (softmax always, the others when no autograd graph is recorded); every other
+call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
+the single-kernel path off.
 """
 import math
 
 import torch
 
+from . import fused
 from .pam_ops import bmm, div, exp2, linear, log2, mul, pow
 
 __all__ = ["mean", "softmax", "logsumexp", "log_softmax", "layer_norm", "LayerNorm",
            "conv2d", "conv2d_group", "Conv2d"]
 
 _LOG2_E = math.log2(math.e)
+fused_rows = True
+
+
+def _fused(x, dim, use_kernel, *grad_sources):
+    """True when the call can run as one kernel; grad_sources empty means a gradient is available."""
+    if not (fused_rows and use_kernel and fused.fusable(x, dim)):
+        return False
+    return not grad_sources or fused.can_skip_graph(*grad_sources)
 
 
 def _pam_kwargs(offset, approx_bwd, use_kernel):
@@ -26,6 +40,8 @@ def mean(input, dim=None, keepdim=False, *, dtype=None, offset=None, approx_bwd=
         dim = tuple(range(input.dim()))
     elif isinstance(dim, int):
         dim = (dim,)
+    if dtype in (None, torch.float32) and _fused(input, dim, use_kernel, input):
+        return fused.mean_last(input, keepdim, offset)
     count = math.prod(input.shape[d] for d in dim)
     total = torch.sum(input, dim=dim, keepdim=keepdim, dtype=dtype)
     return div(total, count, **_pam_kwargs(offset, approx_bwd, use_kernel))
@@ -44,6 +60,8 @@ def _scaled_exp2(x, kw, masked):
 
 def softmax(x, dim=None, *, offset=None, approx_bwd=False, use_kernel=True):
     """pam/pam_ops.py:305-328; -inf inputs give exactly zero weight."""
+    if _fused(x, dim, use_kernel):
+        return fused.softmax(x, offset, approx_bwd)
     kw = _pam_kwargs(offset, approx_bwd, use_kernel)
     masked = x == float("-inf")
     weights, _ = _scaled_exp2(x, kw, masked)
@@ -55,6 +73,8 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
     """pam/pam_ops.py:331-342; inputs must be finite."""
     kw = _pam_kwargs(offset, approx_bwd, use_kernel)
     assert x.isfinite().all()
+    if _fused(x, dim, use_kernel, x):
+        return fused.logsumexp(x, keepdim, offset)
     weights, shift = _scaled_exp2(x, kw, None)
     total = torch.sum(weights, dim=dim, keepdim=keepdim)
     return div(shift + log2(total, **kw), _LOG2_E, **kw)
@@ -62,6 +82,9 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
 
 def log_softmax(x, dim=None, *, offset=None, approx_bwd=False, use_kernel=True):
     """pam/pam_ops.py:345-347"""
+    if _fused(x, dim, use_kernel, x):
+        assert x.isfinite().all()
+        return fused.log_softmax(x, offset)
     return x - logsumexp(x, dim=dim, keepdim=True, **_pam_kwargs(offset, approx_bwd, use_kernel))
 
 
@@ -73,6 +96,9 @@ def layer_norm(x, normalized_shape, weight=None, bias=None, eps=1e-05, *,
     if isinstance(normalized_shape, int):
         normalized_shape = (normalized_shape,)
     assert x.shape[-len(normalized_shape):] == normalized_shape
+    if _fused(x, -1, use_kernel, x, weight, bias) and all(
+            t is None or (t.is_cuda and t.dtype == torch.float32) for t in (weight, bias)):
+        return fused.layer_norm(x, math.prod(normalized_shape), weight, bias, eps, offset)
     rows = x.reshape((-1, math.prod(normalized_shape)))
     centred = rows - mean(rows, dim=-1, keepdim=True, **kw)
     variance = mean(mul(centred, centred, **kw), dim=-1, keepdim=True, **kw)

@@ -1,0 +1,344 @@
+// Row-wise compositions of the piecewise-affine primitives as single kernels for gfx950:
+// softmax (forward and backward), logsumexp / log_softmax, layer_norm and the row mean.
+//
+// Each is, element for element, the chain of primitive calls that the reference's op
+// library makes (pam/pam_ops.py:288-378) with its autograd formulas
+// (pam/cuda_bindings.py:27-57, 66-97, 210-239); what is fused away is the traffic: the
+// unfused chain moves every intermediate through HBM (68 B per element for softmax),
+// here a row is read once from HBM (again from cache for the second sweep) and written
+// once.  One wavefront owns a row: lane l takes the elements l, l + 64, l + 128, ...
+//
+// The reference leaves the order of its row sums to torch.sum.  Here the order is fixed:
+// lane l adds its elements in ascending order starting from +0, then the 64 partial sums
+// are combined by a butterfly, p[l] = p[l] + p[l ^ s] for s = 32, 16, 8, 4, 2, 1.
+// All kernels are HBM-bound streams: 12 B/element for softmax forward (4 for the global
+// maximum sweep, 4 in, 4 out), 12 for its backward, 8 for layer_norm and log_softmax.
+#include <math.h>
+
+#include "pam_common.h"
+#include "pam_device.h"
+
+using namespace pamdev;
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
+constexpr int kMaxPartials = 1024;
+constexpr float kLog2E = (float)1.4426950408889634;      // math.log2(math.e) rounded to fp32 (pam/pam_ops.py:311)
+constexpr float kLn2 = (float)0.6931471805599453;        // math.log(2.0) rounded to fp32 (pam/cuda_bindings.py:235-236)
+
+struct Offset { float off; bool has; };
+
+__device__ __forceinline__ float wave_sum(float p)
+{
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) p = p + __shfl_xor(p, s, 64);
+    return p;
+}
+
+// maximum that propagates NaN, as torch.max does
+struct MaxNan {
+    float mx = u2f(0xff800000u); bool nan = false;
+    __device__ __forceinline__ void take(float v) { if (v != v) nan = true; else mx = fmaxf(mx, v); }
+    __device__ __forceinline__ void merge_wave()
+    {
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) mx = fmaxf(mx, __shfl_xor(mx, s, 64));
+        nan = __ballot(nan) != 0ull;
+    }
+    __device__ __forceinline__ float value() const { return nan ? u2f(kQNaN) : mx; }
+};
+
+// x log2(e) as a PAM product; -inf (attention masks) stays -inf (pam/pam_ops.py:312-317)
+__device__ __forceinline__ float scaled(float x, Offset o, bool mask_inf)
+{
+    if (mask_inf && f2u(x) == 0xff800000u) return x;
+    return pam_mul_off(x, kLog2E, o.off, o.has);
+}
+
+// exp2 through the kernel entry point of that name: pa_exp2(t (*) log2(2)) (pam/cuda_bindings.py:246)
+__device__ __forceinline__ float exp2_op(float t, Offset o) { return pa_exp2(pam_mul_off(t, 1.0f, o.off, o.has)); }
+// log2 likewise: pa_log2(v) (/) log2(2)
+__device__ __forceinline__ float log2_op(float v, Offset o) { return pad_div_off(pa_log2(v), 1.0f, o.off, o.has); }
+
+// ---------------------------------------------------------------- global maximum of the scaled input
+__global__ __launch_bounds__(kThreads) void scaled_max_kernel(const float* __restrict__ x, size_t n, Offset o, int mask_inf,
+                                                             float* __restrict__ partial)
+{
+    MaxNan m;
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += step) m.take(scaled(x[i], o, mask_inf != 0));
+    m.merge_wave();
+    __shared__ float smx[kWaves]; __shared__ int snan[kWaves];
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    if (lane == 0) { smx[wave] = m.mx; snan[wave] = m.nan; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        MaxNan t;
+        for (int w = 0; w < kWaves; ++w) { t.mx = fmaxf(t.mx, smx[w]); t.nan |= snan[w] != 0; }
+        partial[blockIdx.x] = t.value();
+    }
+}
+
+// every wavefront folds the per-block maxima itself (at most 4 KiB, cache resident): floor(max)
+__device__ __forceinline__ float fold_shift(const float* __restrict__ partial, int count, int lane)
+{
+    MaxNan m;
+    for (int i = lane; i < count; i += 64) m.take(partial[i]);
+    m.merge_wave();
+    return floorf(m.value());
+}
+
+// ---------------------------------------------------------------- softmax forward (pam/pam_ops.py:305-328)
+__device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
+{
+    if (f2u(x) == 0xff800000u) return 0.0f;
+    return exp2_op(scaled(x, o, false) - shift, o);
+}
+
+__global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                              float* __restrict__ row_sum, float* __restrict__ shift_out,
+                                                              long rows, long n, Offset o,
+                                                              const float* __restrict__ partial, int partials)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float shift = fold_shift(partial, partials, lane);
+    if (wave == 0 && lane == 0) *shift_out = shift;
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n; float* yr = y + r * n;
+        float p = 0.0f;
+        for (long i = lane; i < n; i += 64) p = p + softmax_weight(xr[i], shift, o);
+        const float total = wave_sum(p);
+        for (long i = lane; i < n; i += 64) yr[i] = pad_div_off(softmax_weight(xr[i], shift, o), total, o.off, o.has);
+        if (lane == 0) row_sum[r] = total;
+    }
+}
+
+// ---------------------------------------------------------------- softmax backward
+// The chain of pad, sum, where, exp2, subtract, where, mul gradients in the order autograd
+// applies them (pam/cuda_bindings.py:78-97, 224-239, 43-57).
+struct Approx { bool a, b, e; };
+
+__device__ __forceinline__ float softmax_dsum_term(float e, float total, float g, Offset o, Approx ap)
+{
+    if (ap.b) return -pam_mul_off(pad_div_off(pad_div_off(e, total, o.off, o.has), total, o.off, o.has), g, o.off, o.has);
+    return pad_div_bwd(e, total, g, o.off, o.has);
+}
+
+__global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                              const float* __restrict__ row_sum, const float* __restrict__ shift_in,
+                                                              float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float shift = *shift_in;
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n; const float* gr = dy + r * n; float* dr = dx + r * n;
+        const float total = row_sum[r];
+        const float inv = pad_div_off(1.0f, total, o.off, o.has);
+        float p = 0.0f;
+        for (long i = lane; i < n; i += 64) p = p + softmax_dsum_term(softmax_weight(xr[i], shift, o), total, gr[i], o, ap);
+        const float dtotal = wave_sum(p);
+        for (long i = lane; i < n; i += 64) {
+            const float xv = xr[i], g = gr[i];
+            const bool masked = f2u(xv) == 0xff800000u;
+            const float e = softmax_weight(xv, shift, o);
+            float de = ap.a ? pam_mul_off(inv, g, o.off, o.has) : pam_mul_bwd(e, inv, g, 1.0f, false);
+            de = de + dtotal;
+            if (masked) de = 0.0f;
+            const float t = scaled(xv, o, true) - shift;
+            float dt;
+            if (ap.e) {
+                float grad = pam_mul_off(exp2_op(t, o), kLn2, o.off, o.has);
+                dt = pam_mul_off(grad, de, o.off, o.has);
+            } else {
+                dt = pam_mul_bwd(t, 1.0f, pa_exp2_bwd(pam_mul_off(t, 1.0f, o.off, o.has), de), o.off, o.has);
+            }
+            if (masked) dt = 0.0f;
+            dr[i] = ap.a ? pam_mul_off(dt, kLog2E, o.off, o.has) : pam_mul_bwd(xv, kLog2E, dt, o.off, o.has);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- logsumexp and log_softmax (pam/pam_ops.py:331-347)
+__global__ __launch_bounds__(kThreads) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
+                                                            float* __restrict__ y, long rows, long n, Offset o,
+                                                            const float* __restrict__ partial, int partials)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float shift = fold_shift(partial, partials, lane);
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n;
+        float p = 0.0f;
+        for (long i = lane; i < n; i += 64) p = p + exp2_op(scaled(xr[i], o, false) - shift, o);
+        const float total = wave_sum(p);
+        const float out = pad_div_off(shift + log2_op(total, o), kLog2E, o.off, o.has);
+        if (lse && lane == 0) lse[r] = out;
+        if (y) {
+            float* yr = y + r * n;
+            for (long i = lane; i < n; i += 64) yr[i] = xr[i] - out;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- row mean (pam/pam_ops.py:288-302)
+__global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                           long rows, long n, Offset o)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float count = (float)n;
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n;
+        float p = 0.0f;
+        for (long i = lane; i < n; i += 64) p = p + xr[i];
+        const float total = wave_sum(p);
+        if (lane == 0) y[r] = pad_div_off(total, count, o.off, o.has);
+    }
+}
+
+// ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
+__global__ __launch_bounds__(kThreads) void layer_norm_fwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                                 const float* __restrict__ bias, float* __restrict__ y,
+                                                                 long rows, long n, float eps, Offset o)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float count = (float)n;
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n; float* yr = y + r * n;
+        float p = 0.0f;
+        for (long i = lane; i < n; i += 64) p = p + xr[i];
+        const float mu = pad_div_off(wave_sum(p), count, o.off, o.has);
+        p = 0.0f;
+        for (long i = lane; i < n; i += 64) { float c = xr[i] - mu; p = p + pam_mul_off(c, c, o.off, o.has); }
+        const float var = pad_div_off(wave_sum(p), count, o.off, o.has);
+        const float v = var + eps;
+        // pow(v, 0.5) = exp2(log2(v) (*) 0.5), zero at zero (pam/pam_ops.py:70-79)
+        const float denom = v == 0.0f ? 0.0f : exp2_op(pam_mul_off(log2_op(v, o), 0.5f, o.off, o.has), o);
+        for (long i = lane; i < n; i += 64) {
+            float out = pad_div_off(xr[i] - mu, denom, o.off, o.has);
+            if (weight) out = pam_mul_off(out, weight[i], o.off, o.has);
+            if (bias) out = out + bias[i];
+            yr[i] = out;
+        }
+    }
+}
+
+int g_cus = 0;
+int cu_count()
+{
+    if (g_cus == 0) {
+        int dev = 0; hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+            g_cus = prop.multiProcessorCount;
+        else g_cus = 256;
+    }
+    return g_cus;
+}
+
+// one wavefront per row, at most 16 wavefronts per SIMD's worth of work-groups in flight
+unsigned row_grid(long rows)
+{
+    long blocks = (rows + kWaves - 1) / kWaves;
+    long cap = (long)cu_count() * 16;
+    return (unsigned)(blocks < cap ? (blocks < 1 ? 1 : blocks) : cap);
+}
+
+int check_rows(const char* what, long rows, long n)
+{
+    if (rows < 0 || n < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: negative size", what);
+    if (n > (1L << 30) || rows > (1L << 40)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: size out of range", what);
+    return PAM_HIP_OK;
+}
+
+int launch_max(const char* what, const float* x, long rows, long n, Offset o, int mask_inf, void* workspace,
+               size_t workspace_bytes, hipStream_t st, int* partials)
+{
+    if (!workspace || workspace_bytes < pam_hip_rowop_workspace_bytes())
+        return pamhost::fail(PAM_HIP_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", what, pam_hip_rowop_workspace_bytes());
+    size_t total = (size_t)rows * (size_t)n;
+    size_t blocks = (total + (size_t)kThreads * 16 - 1) / ((size_t)kThreads * 16);
+    if (blocks > (size_t)kMaxPartials) blocks = kMaxPartials;
+    if (blocks < 1) blocks = 1;
+    *partials = (int)blocks;
+    hipLaunchKernelGGL(scaled_max_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, x, total, o, mask_inf, (float*)workspace);
+    return pamhost::check_launch(what);
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t pam_hip_rowop_workspace_bytes(void) { return (size_t)kMaxPartials * sizeof(float); }
+
+int pam_hip_softmax_fwd(const float* x, float* y, float* row_sum, float* shift, long rows, long n, float offset,
+                        void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_rows("softmax_fwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0 || n == 0) return PAM_HIP_OK;
+    if (!x || !y || !row_sum || !shift) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "softmax_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
+    rc = launch_max("softmax_fwd", x, rows, n, o, 1, workspace, workspace_bytes, st, &partials);
+    if (rc != PAM_HIP_OK) return rc;
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, st, x, y, row_sum, shift, rows, n, o,
+                       (const float*)workspace, partials);
+    return pamhost::check_launch("softmax_fwd");
+}
+
+int pam_hip_softmax_bwd(const float* x, const float* dy, const float* row_sum, const float* shift, float* dx,
+                        long rows, long n, float offset, int approx_a, int approx_b, int approx_exp, void* stream)
+{
+    int rc = check_rows("softmax_bwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0 || n == 0) return PAM_HIP_OK;
+    if (!x || !dy || !row_sum || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "softmax_bwd: null pointer");
+    Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
+    hipLaunchKernelGGL(softmax_bwd_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream,
+                       x, dy, row_sum, shift, dx, rows, n, o, ap);
+    return pamhost::check_launch("softmax_bwd");
+}
+
+int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, long rows, long n, float offset,
+                          void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_rows("logsumexp_fwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0 || n == 0) return PAM_HIP_OK;
+    if (!x || (!lse && !log_softmax)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
+    rc = launch_max("logsumexp_fwd", x, rows, n, o, 0, workspace, workspace_bytes, st, &partials);
+    if (rc != PAM_HIP_OK) return rc;
+    hipLaunchKernelGGL(logsumexp_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, st, x, lse, log_softmax, rows, n, o,
+                       (const float*)workspace, partials);
+    return pamhost::check_launch("logsumexp_fwd");
+}
+
+int pam_hip_row_mean_fwd(const float* x, float* y, long rows, long n, float offset, void* stream)
+{
+    int rc = check_rows("row_mean_fwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0) return PAM_HIP_OK;
+    if (!y || (n > 0 && !x)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "row_mean_fwd: null pointer");
+    hipLaunchKernelGGL(row_mean_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, y, rows, n,
+                       Offset{offset, offset != 1.0f});
+    return pamhost::check_launch("row_mean_fwd");
+}
+
+int pam_hip_layer_norm_fwd(const float* x, const float* weight, const float* bias, float* y, long rows, long n,
+                           float eps, float offset, void* stream)
+{
+    int rc = check_rows("layer_norm_fwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0 || n == 0) return PAM_HIP_OK;
+    if (!x || !y) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_fwd: null pointer");
+    hipLaunchKernelGGL(layer_norm_fwd_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, weight, bias, y,
+                       rows, n, eps, Offset{offset, offset != 1.0f});
+    return pamhost::check_launch("layer_norm_fwd");
+}
+
+}  // extern "C"

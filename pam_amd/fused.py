@@ -1,0 +1,92 @@
+"""Row-wise compositions as single kernels: softmax (with its gradient), logsumexp,
+log_softmax, the mean over the last dimension and layer_norm.
+
+Each computes, element for element, what the compositions of `pam_amd.composites` compute
+from the primitive kernels (the reference's pam/pam_ops.py:288-378), in one sweep over the
+rows instead of five to fifteen elementwise launches.  The only difference is the order of
+the row sums, which the reference leaves to torch.sum and the kernels fix.
+
+`row_kernels` is the kernel object; tests may swap it for another object with the same
+five methods.  `fusable` says whether a call can take this path: float32 GPU tensor,
+contiguous, reduced dimension last, not empty.
+"""
+import torch
+
+from ._abi import HipRowKernels
+from .cuda_bindings import _both, _offset_value
+
+row_kernels = HipRowKernels()
+
+
+def fusable(x, dim):
+    if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.float32):
+        return False
+    if x.dim() < 1 or x.numel() == 0 or not x.is_contiguous():
+        return False
+    if isinstance(dim, (tuple, list)):
+        if len(dim) != 1:
+            return False
+        dim = dim[0]
+    return isinstance(dim, int) and dim in (-1, x.dim() - 1)
+
+
+def _wants_grad(*tensors):
+    return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
+class softmax_autograd(torch.autograd.Function):
+    """softmax over the last dimension; the gradient is the chain of the primitives'
+    gradients (pam/cuda_bindings.py:43-57, 78-97, 224-239) in one kernel."""
+
+    @staticmethod
+    def forward(ctx, x, offset=None, approx_bwd=False):
+        ctx.offset = _offset_value(offset)
+        ctx.approx_bwd = approx_bwd
+        rows = x.reshape(-1, x.shape[-1])
+        y, row_sum, shift = row_kernels.softmax_fwd(rows, ctx.offset)
+        ctx.save_for_backward(rows, row_sum, shift)
+        return y.view(x.shape)
+
+    @staticmethod
+    def backward(ctx, grad):
+        rows, row_sum, shift = ctx.saved_tensors
+        approx_a, approx_b = _both(ctx.approx_bwd)
+        # exp2's backward tests the flag's truth value, so a pair counts as set
+        # (pam/cuda_bindings.py:227)
+        approx_exp = bool(ctx.approx_bwd)
+        g = grad.contiguous().view(rows.shape)
+        dx = row_kernels.softmax_bwd(rows, g, row_sum, shift, ctx.offset, approx_a, approx_b, approx_exp)
+        return dx.view(grad.shape), None, None
+
+
+def softmax(x, offset=None, approx_bwd=False):
+    return softmax_autograd.apply(x, offset, approx_bwd)
+
+
+# The remaining fused forwards have no fused gradient: they serve calls that record no
+# graph, and `composites` keeps the unfused chain for calls that do.
+
+def can_skip_graph(*tensors):
+    return not _wants_grad(*tensors)
+
+
+def logsumexp(x, keepdim, offset=None):
+    lse, _ = row_kernels.logsumexp_fwd(x.reshape(-1, x.shape[-1]), _offset_value(offset), True, False)
+    shape = x.shape[:-1] + ((1,) if keepdim else ())
+    return lse.view(shape)
+
+
+def log_softmax(x, offset=None):
+    _, y = row_kernels.logsumexp_fwd(x.reshape(-1, x.shape[-1]), _offset_value(offset), False, True)
+    return y.view(x.shape)
+
+
+def mean_last(x, keepdim, offset=None):
+    y = row_kernels.row_mean_fwd(x.reshape(-1, x.shape[-1]), _offset_value(offset))
+    return y.view(x.shape[:-1] + ((1,) if keepdim else ()))
+
+
+def layer_norm(x, n, weight, bias, eps, offset=None):
+    w = None if weight is None else weight.detach().contiguous().view(-1)
+    b = None if bias is None else bias.detach().contiguous().view(-1)
+    return row_kernels.layer_norm_fwd(x.reshape(-1, n), w, b, eps, _offset_value(offset)).view(x.shape)

@@ -1,0 +1,298 @@
+"""Single-kernel softmax / logsumexp / log_softmax / mean / layer_norm.
+
+CPU: the oracle's fused restatements are pinned against the chain of primitive calls the
+reference makes (pam/pam_ops.py:288-378), written out here from the already pinned oracle
+primitives with the kernels' row-sum order restated in numpy: bit for bit.  The softmax
+gradient is pinned twice: against the primitives' backward formulas chained by hand, and
+against torch autograd running the unfused composition over the oracle-backed kernel object
+(there the row sums are torch's, so the comparison is to summation-order noise).
+GPU: the HIP kernels against the oracle's fused restatements, bit for bit.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import pam_amd
+from pam_amd import composites, cuda_bindings, pam_ops
+from _util import assert_same_bits, same_bits
+from test_host_api import OracleKernels
+
+C = np.float32(math.log2(math.e))
+LN2 = np.float32(math.log(2.0))
+OFF = 1.0552
+
+
+def fixed_sum(v):
+    """Row sums in the kernels' order: 64 strided partial sums from +0, then a butterfly."""
+    v = np.asarray(v, dtype=np.float32)
+    rows, n = v.shape
+    pad = (-n) % 64
+    if pad:
+        v = np.concatenate([v, np.zeros((rows, pad), np.float32)], axis=1)     # adding +0 changes nothing
+    p = np.zeros((rows, 64), np.float32)
+    for j in range(v.shape[1] // 64):
+        p = (p + v[:, 64 * j:64 * j + 64]).astype(np.float32)
+    lanes = np.arange(64)
+    for s in (32, 16, 8, 4, 2, 1):
+        p = (p + p[:, lanes ^ s]).astype(np.float32)
+    return p[:, 0]
+
+
+def rows_case(seed, rows, n, scale=3.0, masks=True):
+    rng = np.random.RandomState(seed)
+    x = (rng.standard_normal((rows, n)) * scale).astype(np.float32)
+    if masks and n > 2:
+        x[rng.randint(rows), rng.randint(n)] = -np.inf
+        x[rng.randint(rows), : n // 2] = -np.inf
+    return x
+
+
+# ------------------------------------------------------------------ the reference's chains, from oracle primitives
+def softmax_chain(o, x, off):
+    neg = np.isneginf(x)
+    s = np.where(neg, -np.inf, o.pam(x, C, off)).astype(np.float32)
+    shift = np.floor(s.max())
+    t = (s - shift).astype(np.float32)
+    e = np.where(neg, 0, o.pa_exp(t, 2.0, off)).astype(np.float32)
+    total = fixed_sum(e)[:, None]
+    return o.pad(e, total, off), dict(neg=neg, t=t, e=e, total=total, shift=shift)
+
+
+def softmax_grad_chain(o, x, g, off, approx):
+    """pad -> sum -> where -> exp2 -> subtract -> where -> mul, each with the backward formula of
+    its autograd Function (pam/cuda_bindings.py:43-57, 78-97, 224-239)."""
+    approx_a, approx_b, approx_e = approx
+    _, f = softmax_chain(o, x, off)
+    neg, t, e, total = f["neg"], f["t"], f["e"], np.broadcast_to(f["total"], x.shape)
+    inv = o.pad(np.ones_like(total), total, off)
+    d_e = o.pam(inv, g, off) if approx_a else o.pam_bwd(e, inv, g, None)
+    if approx_b:
+        d_total_full = (-o.pam(o.pad(o.pad(e, total, off), total, off), g, off)).astype(np.float32)
+    else:
+        d_total_full = o.pad_bwd(e, total, g, off)
+    d_total = fixed_sum(d_total_full)[:, None]
+    d_e = np.where(neg, 0, (d_e + d_total).astype(np.float32)).astype(np.float32)
+    if approx_e:
+        d_t = o.pam(o.pam(o.pa_exp(t, 2.0, off), LN2, off), d_e, off)
+    else:
+        d_t = o.pa_exp_bwd(t, d_e, 2.0, off)
+    d_s = np.where(neg, 0, d_t).astype(np.float32)
+    return o.pam(d_s, C, off) if approx_a else o.pam_bwd(x, C, d_s, off)
+
+
+def logsumexp_chain(o, x, off):
+    s = o.pam(x, C, off)
+    shift = np.floor(s.max())
+    e = o.pa_exp((s - shift).astype(np.float32), 2.0, off)
+    total = fixed_sum(e)
+    return o.pad((shift + o.pa_log(total, 2.0, off)).astype(np.float32), C, off)
+
+
+def layer_norm_chain(o, x, w, b, eps, off):
+    n = np.float32(x.shape[1])
+    mu = o.pad(fixed_sum(x)[:, None], n, off)
+    cen = (x - mu).astype(np.float32)
+    var = o.pad(fixed_sum(o.pam(cen, cen, off))[:, None], n, off)
+    v = (var + np.float32(eps)).astype(np.float32)
+    root = np.where(v == 0, 0, o.pa_exp(o.pam(o.pa_log(v, 2.0, off), np.float32(0.5), off), 2.0, off)).astype(np.float32)
+    out = o.pad(cen, root, off)
+    if w is not None:
+        out = o.pam(out, w, off)
+    if b is not None:
+        out = (out + b).astype(np.float32)
+    return out
+
+
+# ------------------------------------------------------------------ CPU: oracle fused == chain
+@pytest.mark.parametrize("off", [None, OFF])
+@pytest.mark.parametrize("rows,n", [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (6, 197), (2, 1000)])
+def test_oracle_softmax_is_the_chain(oracle, rows, n, off):
+    x = rows_case(rows * 1000 + n, rows, n)
+    y, row_sum, shift = oracle.softmax_fwd(x, off)
+    want, f = softmax_chain(oracle, x, off)
+    assert_same_bits(y, want, "softmax")
+    assert_same_bits(row_sum, f["total"][:, 0], "row sums")
+    assert_same_bits(shift, f["shift"], "shift")
+    g = np.random.RandomState(7).standard_normal(x.shape).astype(np.float32)
+    for approx in [(False, False, False), (True, True, True), (True, False, True), (False, True, True)]:
+        got = oracle.softmax_bwd(x, g, row_sum, shift, off, approx)
+        assert_same_bits(got, softmax_grad_chain(oracle, x, g, off, approx), f"softmax gradient approx={approx}")
+
+
+def test_oracle_softmax_special_rows(oracle):
+    x = rows_case(3, 6, 40, masks=False)
+    x[0, :] = -np.inf                       # fully masked row: 0 (/) 0
+    x[1, 3] = np.nan
+    y, _, _ = oracle.softmax_fwd(x)
+    assert np.isnan(y).all()                # the NaN reaches the global shift, as in the reference's chain
+    x[1, 3] = 0.5
+    y, row_sum, _ = oracle.softmax_fwd(x)
+    assert np.isnan(y[0]).all() and row_sum[0] == 0 and np.isfinite(y[1:]).all()
+    assert_same_bits(y, softmax_chain(oracle, x, None)[0], "masked row")
+    assert np.abs(y[1:].sum(-1) - 1).max() < 0.1
+
+
+@pytest.mark.parametrize("off", [None, OFF])
+def test_oracle_logsumexp_mean_layer_norm_are_the_chains(oracle, off):
+    for rows, n in [(1, 1), (3, 7), (4, 64), (5, 192), (2, 513)]:
+        x = rows_case(rows * 77 + n, rows, n, masks=False)
+        want = logsumexp_chain(oracle, x, off)
+        lse, ls = oracle.logsumexp_fwd(x, off, with_log_softmax=True)
+        assert_same_bits(lse, want, "logsumexp")
+        assert_same_bits(ls, (x - want[:, None]).astype(np.float32), "log_softmax")
+        assert_same_bits(oracle.row_mean_fwd(x, off), oracle.pad(fixed_sum(x), np.float32(n), off), "mean")
+        rng = np.random.RandomState(n)
+        w, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+        for ww, bb in [(None, None), (w, None), (w, b)]:
+            assert_same_bits(oracle.layer_norm_fwd(x, ww, bb, 1e-5, off), layer_norm_chain(oracle, x, ww, bb, 1e-5, off),
+                             "layer_norm")
+    const = np.full((2, 8), 3.0, np.float32)              # zero variance: the power's zero branch is not taken (eps)
+    assert np.isfinite(oracle.layer_norm_fwd(const)).all()
+    assert_same_bits(oracle.layer_norm_fwd(const, eps=0.0), np.full((2, 8), np.nan, np.float32), "0 (/) 0")
+
+
+def test_fixed_order_sum_is_exact_where_sums_are(oracle):
+    """Rows whose sums are exact in fp32 give the same result in any order: ties the fixed
+    order to torch's on such rows."""
+    rng = np.random.RandomState(5)
+    x = (rng.randint(-64, 64, size=(6, 300)) / 8.0).astype(np.float32)
+    assert_same_bits(fixed_sum(x), x.sum(-1, dtype=np.float64).astype(np.float32), "exact sums")
+    assert_same_bits(oracle.row_mean_fwd(x), oracle.pad(x.sum(-1, dtype=np.float64).astype(np.float32), np.float32(300)), "mean")
+
+
+@pytest.fixture()
+def on_cpu(oracle, monkeypatch):
+    monkeypatch.setattr(cuda_bindings, "cuda_kernels", OracleKernels(oracle))
+    monkeypatch.setattr(pam_ops, "_require_kernel", lambda t, use_kernel: None)
+    return oracle
+
+
+@pytest.mark.parametrize("approx", [False, True, (True, False)])
+def test_softmax_gradient_chain_is_what_autograd_does(on_cpu, approx):
+    """torch autograd over the unfused composition (oracle-backed kernels, CPU) against the
+    fused restatement: same formulas, torch's summation order instead of the fixed one."""
+    o = on_cpu
+    x = rows_case(11, 7, 33)
+    g = np.random.RandomState(12).standard_normal(x.shape).astype(np.float32)
+    for off in (None, OFF):
+        xt = torch.from_numpy(x.copy()).requires_grad_()
+        y = composites.softmax(xt, dim=-1, offset=off, approx_bwd=approx)
+        y.backward(torch.from_numpy(g))
+        flags = (approx, approx, approx) if isinstance(approx, bool) else (approx[0], approx[1], True)
+        yo, row_sum, shift = o.softmax_fwd(x, off)
+        got = o.softmax_bwd(x, g, row_sum, shift, off, flags)
+        want = xt.grad.numpy()
+        assert np.allclose(yo, y.detach().numpy(), rtol=2e-6, atol=1e-7)
+        scale = np.abs(want).max()
+        assert np.isfinite(want).all() and np.abs(got - want).max() <= 5e-6 * scale, (np.abs(got - want).max(), scale)
+        assert (got[np.isneginf(x)] == 0).all()
+
+
+# ------------------------------------------------------------------ GPU: HIP kernels == oracle fused
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("off", [None, OFF])
+def test_gpu_softmax_forward_backward(oracle, off):
+    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (64, 197), (2, 1000), (300, 32), (5, 4097)]:
+        x = rows_case(rows * 1000 + n, rows, n)
+        g = np.random.RandomState(n).standard_normal(x.shape).astype(np.float32)
+        want, row_sum, shift = oracle.softmax_fwd(x, off)
+        for approx in (False, True, (True, False), (False, True)):
+            xt = _dev(x).requires_grad_()
+            y = pam_amd.softmax(xt, dim=-1, offset=off, approx_bwd=approx)
+            assert_same_bits(y.detach().cpu().numpy(), want, f"softmax {rows}x{n}")
+            y.backward(_dev(g))
+            flags = (approx, approx, approx) if isinstance(approx, bool) else (approx[0], approx[1], True)
+            assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, off, flags),
+                             f"softmax gradient {rows}x{n} approx={approx}")
+
+
+@pytest.mark.gpu
+def test_gpu_softmax_matches_unfused_composition(oracle):
+    """The single kernel against the chain of primitive kernels on the same device: equal up to
+    the order of the row sums; leading dimensions and the module-level switch."""
+    x = rows_case(21, 12 * 7, 50).reshape(12, 7, 50)
+    g = np.random.RandomState(3).standard_normal(x.shape).astype(np.float32)
+    res = {}
+    for fused_on in (True, False):
+        composites.fused_rows = fused_on
+        try:
+            xt = _dev(x).requires_grad_()
+            y = pam_amd.softmax(xt, dim=-1, approx_bwd=True)
+            y.backward(_dev(g))
+            res[fused_on] = (y.detach().cpu().numpy(), xt.grad.cpu().numpy())
+        finally:
+            composites.fused_rows = True
+    assert np.allclose(res[True][0], res[False][0], rtol=2e-6, atol=1e-7)
+    scale = np.abs(res[False][1]).max()
+    assert np.abs(res[True][1] - res[False][1]).max() <= 5e-6 * scale
+    # a reduction over another dimension keeps the unfused chain
+    y0 = pam_amd.softmax(_dev(x), dim=1)
+    assert y0.shape == x.shape and torch.isfinite(y0[~torch.isnan(y0)]).all()
+
+
+@pytest.mark.gpu
+def test_gpu_softmax_special_values(oracle):
+    x = rows_case(3, 6, 40, masks=False)
+    x[0, :] = -np.inf
+    x[2, 5] = 3.0e38
+    x[3, 1] = 1e-40
+    x[4, 2] = 0.0
+    want, row_sum, shift = oracle.softmax_fwd(x)
+    assert_same_bits(pam_amd.softmax(_dev(x), dim=-1).cpu().numpy(), want, "special values")
+    x[1, 3] = np.nan
+    assert torch.isnan(pam_amd.softmax(_dev(x), dim=-1)).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("off", [None, OFF])
+def test_gpu_logsumexp_mean_layer_norm(oracle, off):
+    for rows, n in [(1, 1), (3, 7), (4, 64), (50, 192), (2, 513), (33, 512), (3, 10000)]:
+        x = rows_case(rows * 77 + n, rows, n, masks=False)
+        xt = _dev(x)
+        lse, ls = oracle.logsumexp_fwd(x, off, with_log_softmax=True)
+        assert_same_bits(pam_amd.logsumexp(xt, dim=-1, offset=off).cpu().numpy(), lse, "logsumexp")
+        assert pam_amd.logsumexp(xt, dim=-1, keepdim=True, offset=off).shape == (rows, 1)
+        assert_same_bits(pam_amd.log_softmax(xt, dim=-1, offset=off).cpu().numpy(), ls, "log_softmax")
+        assert_same_bits(pam_amd.mean(xt, dim=-1, offset=off).cpu().numpy(), oracle.row_mean_fwd(x, off), "mean")
+        rng = np.random.RandomState(n)
+        w, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+        for ww, bb in [(None, None), (w, None), (w, b)]:
+            got = pam_amd.layer_norm(xt, n, None if ww is None else _dev(ww), None if bb is None else _dev(bb), offset=off)
+            assert_same_bits(got.cpu().numpy(), oracle.layer_norm_fwd(x, ww, bb, 1e-5, off), f"layer_norm {rows}x{n}")
+
+
+@pytest.mark.gpu
+def test_gpu_layer_norm_with_graph_keeps_gradients(oracle):
+    """With a graph recorded the unfused chain runs (it carries the gradient); the values agree
+    with the single kernel up to the order of the row sums."""
+    x = rows_case(9, 40, 192, masks=False)
+    ln = pam_amd.LayerNorm(192, approx_bwd=True).cuda()
+    xt = _dev(x).requires_grad_()
+    y = ln(xt)
+    y.sum().backward()
+    assert xt.grad is not None and torch.isfinite(xt.grad).all() and ln.weight.grad is not None
+    with torch.no_grad():
+        y2 = ln(_dev(x))
+    assert_same_bits(y2.cpu().numpy(), oracle.layer_norm_fwd(x, np.ones(192, np.float32), np.zeros(192, np.float32)), "no-grad path")
+    assert np.allclose(y.detach().cpu().numpy(), y2.cpu().numpy(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_gpu_attention_softmax_full_size(oracle):
+    """Attention probabilities at the benchmark's shape, batch 64 x 3 heads x 197 x 197, against the oracle."""
+    rng = np.random.RandomState(0)
+    x = rng.standard_normal((192, 197, 197)).astype(np.float32)
+    g = rng.standard_normal(x.shape).astype(np.float32)
+    xt = _dev(x).requires_grad_()
+    y = pam_amd.softmax(xt, dim=-1, approx_bwd=True)
+    y.backward(_dev(g))
+    want, row_sum, shift = oracle.softmax_fwd(x)
+    assert_same_bits(y.detach().cpu().numpy(), want, "softmax 192x197x197")
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, None, (True, True, True)), "its gradient")
+    assert np.abs(want.sum(-1) - 1).max() < 0.1
