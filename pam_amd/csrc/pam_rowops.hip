@@ -63,12 +63,30 @@ __device__ __forceinline__ float exp2_op(float t, Offset o) { return pa_exp2(pam
 __device__ __forceinline__ float log2_op(float v, Offset o) { return pad_div_off(pa_log2(v), 1.0f, o.off, o.has); }
 
 // ---------------------------------------------------------------- global maximum of the scaled input
-__global__ __launch_bounds__(kThreads) void scaled_max_kernel(const float* __restrict__ x, size_t n, Offset o, int mask_inf,
-                                                             float* __restrict__ partial)
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// 128-bit loads, four in flight per lane; the maximum does not depend on the order
+__global__ __launch_bounds__(kThreads) void scaled_max_kernel(const float* __restrict__ x, size_t n, size_t nvec, Offset o,
+                                                             int mask_inf, float* __restrict__ partial)
 {
     MaxNan m;
-    const size_t step = (size_t)gridDim.x * kThreads;
-    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += step) m.take(scaled(x[i], o, mask_inf != 0));
+    const bool mask = mask_inf != 0;
+    const v4f* xv = reinterpret_cast<const v4f*>(x);
+    const size_t step = (size_t)gridDim.x * (kThreads * 4);
+    for (size_t base = (size_t)blockIdx.x * (kThreads * 4) + threadIdx.x; base < nvec; base += step) {
+        v4f q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) { size_t i = base + (size_t)u * kThreads; if (i < nvec) q[u] = xv[i]; }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (base + (size_t)u * kThreads < nvec) {
+                m.take(scaled(q[u].x, o, mask)); m.take(scaled(q[u].y, o, mask));
+                m.take(scaled(q[u].z, o, mask)); m.take(scaled(q[u].w, o, mask));
+            }
+        }
+    }
+    for (size_t i = nvec * 4 + (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
+        m.take(scaled(x[i], o, mask));
     m.merge_wave();
     __shared__ float smx[kWaves]; __shared__ int snan[kWaves];
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -90,6 +108,33 @@ __device__ __forceinline__ float fold_shift(const float* __restrict__ partial, i
     return floorf(m.value());
 }
 
+// ---------------------------------------------------------------- row access
+// CH > 0: the row fits CH values per lane and is held in registers (one read of x, all loads
+// of a row in flight together); CH == 0: rows of any length, swept twice (the second sweep
+// comes from cache), four loads in flight per lane.
+constexpr float kNegInf = -__builtin_inff();
+
+template <int CH>
+__device__ __forceinline__ void load_row(float (&v)[CH], const float* __restrict__ p, long n, int lane, float fill)
+{
+#pragma unroll
+    for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; v[c] = i < n ? p[i] : fill; }
+}
+
+// p = p + f(x[i]) over the lane's elements in ascending order
+template <class F>
+__device__ __forceinline__ float stream_sum(const float* __restrict__ p, long n, int lane, F f)
+{
+    float acc = 0.0f;
+    long i = lane;
+    for (; i + 192 < n; i += 256) {
+        float a = p[i], b = p[i + 64], c = p[i + 128], d = p[i + 192];
+        acc = acc + f(i, a); acc = acc + f(i + 64, b); acc = acc + f(i + 128, c); acc = acc + f(i + 192, d);
+    }
+    for (; i < n; i += 64) acc = acc + f(i, p[i]);
+    return acc;
+}
+
 // ---------------------------------------------------------------- softmax forward (pam/pam_ops.py:305-328)
 __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
 {
@@ -97,6 +142,7 @@ __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
     return exp2_op(scaled(x, o, false) - shift, o);
 }
 
+template <int CH>
 __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                               float* __restrict__ row_sum, float* __restrict__ shift_out,
                                                               long rows, long n, Offset o,
@@ -108,10 +154,20 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(const float* __re
     if (wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
-        float p = 0.0f;
-        for (long i = lane; i < n; i += 64) p = p + softmax_weight(xr[i], shift, o);
-        const float total = wave_sum(p);
-        for (long i = lane; i < n; i += 64) yr[i] = pad_div_off(softmax_weight(xr[i], shift, o), total, o.off, o.has);
+        float total;
+        if constexpr (CH > 0) {
+            float e[CH];
+            load_row<CH>(e, xr, n, lane, kNegInf);             // the fill has weight zero
+            float p = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { e[c] = softmax_weight(e[c], shift, o); p = p + e[c]; }
+            total = wave_sum(p);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = pad_div_off(e[c], total, o.off, o.has); }
+        } else {
+            total = wave_sum(stream_sum(xr, n, lane, [&](long, float v) { return softmax_weight(v, shift, o); }));
+            for (long i = lane; i < n; i += 64) yr[i] = pad_div_off(softmax_weight(xr[i], shift, o), total, o.off, o.has);
+        }
         if (lane == 0) row_sum[r] = total;
     }
 }
@@ -127,6 +183,21 @@ __device__ __forceinline__ float softmax_dsum_term(float e, float total, float g
     return pad_div_bwd(e, total, g, o.off, o.has);
 }
 
+__device__ __forceinline__ float softmax_dx(float xv, float e, float g, float inv, float dtotal, float shift, Offset o, Approx ap)
+{
+    const bool masked = f2u(xv) == 0xff800000u;
+    float de = ap.a ? pam_mul_off(inv, g, o.off, o.has) : pam_mul_bwd(e, inv, g, 1.0f, false);
+    de = de + dtotal;                                 // quotient's first operand + the broadcast of the sum's
+    if (masked) de = 0.0f;                            // where(x == -inf, 0, exp2(..))
+    const float t = scaled(xv, o, true) - shift;
+    float dt;
+    if (ap.e) dt = pam_mul_off(pam_mul_off(exp2_op(t, o), kLn2, o.off, o.has), de, o.off, o.has);
+    else dt = pam_mul_bwd(t, 1.0f, pa_exp2_bwd(pam_mul_off(t, 1.0f, o.off, o.has), de), o.off, o.has);
+    if (masked) dt = 0.0f;                            // where(x == -inf, -inf, mul(..))
+    return ap.a ? pam_mul_off(dt, kLog2E, o.off, o.has) : pam_mul_bwd(xv, kLog2E, dt, o.off, o.has);
+}
+
+template <int CH>
 __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                               const float* __restrict__ row_sum, const float* __restrict__ shift_in,
                                                               float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
@@ -138,31 +209,35 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const float* __re
         const float* xr = x + r * n; const float* gr = dy + r * n; float* dr = dx + r * n;
         const float total = row_sum[r];
         const float inv = pad_div_off(1.0f, total, o.off, o.has);
-        float p = 0.0f;
-        for (long i = lane; i < n; i += 64) p = p + softmax_dsum_term(softmax_weight(xr[i], shift, o), total, gr[i], o, ap);
-        const float dtotal = wave_sum(p);
-        for (long i = lane; i < n; i += 64) {
-            const float xv = xr[i], g = gr[i];
-            const bool masked = f2u(xv) == 0xff800000u;
-            const float e = softmax_weight(xv, shift, o);
-            float de = ap.a ? pam_mul_off(inv, g, o.off, o.has) : pam_mul_bwd(e, inv, g, 1.0f, false);
-            de = de + dtotal;
-            if (masked) de = 0.0f;
-            const float t = scaled(xv, o, true) - shift;
-            float dt;
-            if (ap.e) {
-                float grad = pam_mul_off(exp2_op(t, o), kLn2, o.off, o.has);
-                dt = pam_mul_off(grad, de, o.off, o.has);
-            } else {
-                dt = pam_mul_bwd(t, 1.0f, pa_exp2_bwd(pam_mul_off(t, 1.0f, o.off, o.has), de), o.off, o.has);
+        if constexpr (CH > 0) {
+            float xv[CH], g[CH], e[CH];
+            load_row<CH>(xv, xr, n, lane, kNegInf);
+            load_row<CH>(g, gr, n, lane, 0.0f);
+            float p = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                e[c] = softmax_weight(xv[c], shift, o);
+                if (lane + 64L * c < n) p = p + softmax_dsum_term(e[c], total, g[c], o, ap);
             }
-            if (masked) dt = 0.0f;
-            dr[i] = ap.a ? pam_mul_off(dt, kLog2E, o.off, o.has) : pam_mul_bwd(xv, kLog2E, dt, o.off, o.has);
+            const float dtotal = wave_sum(p);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                long i = lane + 64L * c;
+                if (i < n) dr[i] = softmax_dx(xv[c], e[c], g[c], inv, dtotal, shift, o, ap);
+            }
+        } else {
+            const float dtotal = wave_sum(stream_sum(xr, n, lane, [&](long i, float v) {
+                return softmax_dsum_term(softmax_weight(v, shift, o), total, gr[i], o, ap); }));
+            for (long i = lane; i < n; i += 64) {
+                const float v = xr[i];
+                dr[i] = softmax_dx(v, softmax_weight(v, shift, o), gr[i], inv, dtotal, shift, o, ap);
+            }
         }
     }
 }
 
 // ---------------------------------------------------------------- logsumexp and log_softmax (pam/pam_ops.py:331-347)
+template <int CH>
 __global__ __launch_bounds__(kThreads) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
                                                             float* __restrict__ y, long rows, long n, Offset o,
                                                             const float* __restrict__ partial, int partials)
@@ -172,14 +247,23 @@ __global__ __launch_bounds__(kThreads) void logsumexp_kernel(const float* __rest
     const float shift = fold_shift(partial, partials, lane);
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
-        float p = 0.0f;
-        for (long i = lane; i < n; i += 64) p = p + exp2_op(scaled(xr[i], o, false) - shift, o);
-        const float total = wave_sum(p);
-        const float out = pad_div_off(shift + log2_op(total, o), kLog2E, o.off, o.has);
-        if (lse && lane == 0) lse[r] = out;
-        if (y) {
-            float* yr = y + r * n;
-            for (long i = lane; i < n; i += 64) yr[i] = xr[i] - out;
+        auto weight = [&](long, float v) { return exp2_op(scaled(v, o, false) - shift, o); };
+        if constexpr (CH > 0) {
+            float xv[CH];
+            load_row<CH>(xv, xr, n, lane, 0.0f);
+            float p = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CH; ++c) if (lane + 64L * c < n) p = p + weight(0, xv[c]);
+            const float out = pad_div_off(shift + log2_op(wave_sum(p), o), kLog2E, o.off, o.has);
+            if (lse && lane == 0) lse[r] = out;
+            if (y) {
+#pragma unroll
+                for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) y[r * n + i] = xv[c] - out; }
+            }
+        } else {
+            const float out = pad_div_off(shift + log2_op(wave_sum(stream_sum(xr, n, lane, weight)), o), kLog2E, o.off, o.has);
+            if (lse && lane == 0) lse[r] = out;
+            if (y) for (long i = lane; i < n; i += 64) y[r * n + i] = xr[i] - out;
         }
     }
 }
@@ -192,15 +276,26 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restr
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float count = (float)n;
     for (long r = wave; r < rows; r += nwaves) {
-        const float* xr = x + r * n;
-        float p = 0.0f;
-        for (long i = lane; i < n; i += 64) p = p + xr[i];
-        const float total = wave_sum(p);
+        const float total = wave_sum(stream_sum(x + r * n, n, lane, [](long, float v) { return v; }));
         if (lane == 0) y[r] = pad_div_off(total, count, o.off, o.has);
     }
 }
 
 // ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
+// pow(v, 0.5) = exp2(log2(v) (*) 0.5), zero at zero (pam/pam_ops.py:70-79)
+__device__ __forceinline__ float root_op(float v, Offset o)
+{ return v == 0.0f ? 0.0f : exp2_op(pam_mul_off(log2_op(v, o), 0.5f, o.off, o.has), o); }
+
+__device__ __forceinline__ float layer_norm_out(float centred, float denom, long i, const float* __restrict__ weight,
+                                               const float* __restrict__ bias, Offset o)
+{
+    float out = pad_div_off(centred, denom, o.off, o.has);
+    if (weight) out = pam_mul_off(out, weight[i], o.off, o.has);
+    if (bias) out = out + bias[i];
+    return out;
+}
+
+template <int CH>
 __global__ __launch_bounds__(kThreads) void layer_norm_fwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
                                                                  const float* __restrict__ bias, float* __restrict__ y,
                                                                  long rows, long n, float eps, Offset o)
@@ -210,23 +305,45 @@ __global__ __launch_bounds__(kThreads) void layer_norm_fwd_kernel(const float* _
     const float count = (float)n;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
-        float p = 0.0f;
-        for (long i = lane; i < n; i += 64) p = p + xr[i];
-        const float mu = pad_div_off(wave_sum(p), count, o.off, o.has);
-        p = 0.0f;
-        for (long i = lane; i < n; i += 64) { float c = xr[i] - mu; p = p + pam_mul_off(c, c, o.off, o.has); }
-        const float var = pad_div_off(wave_sum(p), count, o.off, o.has);
-        const float v = var + eps;
-        // pow(v, 0.5) = exp2(log2(v) (*) 0.5), zero at zero (pam/pam_ops.py:70-79)
-        const float denom = v == 0.0f ? 0.0f : exp2_op(pam_mul_off(log2_op(v, o), 0.5f, o.off, o.has), o);
-        for (long i = lane; i < n; i += 64) {
-            float out = pad_div_off(xr[i] - mu, denom, o.off, o.has);
-            if (weight) out = pam_mul_off(out, weight[i], o.off, o.has);
-            if (bias) out = out + bias[i];
-            yr[i] = out;
+        if constexpr (CH > 0) {
+            float v[CH];
+            load_row<CH>(v, xr, n, lane, 0.0f);
+            float p = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CH; ++c) p = p + v[c];                       // the fill adds +0
+            const float mu = pad_div_off(wave_sum(p), count, o.off, o.has);
+            p = 0.0f;
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { v[c] = v[c] - mu; if (lane + 64L * c < n) p = p + pam_mul_off(v[c], v[c], o.off, o.has); }
+            const float denom = root_op(pad_div_off(wave_sum(p), count, o.off, o.has) + eps, o);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = layer_norm_out(v[c], denom, i, weight, bias, o); }
+        } else {
+            const float mu = pad_div_off(wave_sum(stream_sum(xr, n, lane, [](long, float v) { return v; })), count, o.off, o.has);
+            const float var = pad_div_off(wave_sum(stream_sum(xr, n, lane, [&](long, float v) {
+                float c = v - mu; return pam_mul_off(c, c, o.off, o.has); })), count, o.off, o.has);
+            const float denom = root_op(var + eps, o);
+            for (long i = lane; i < n; i += 64) yr[i] = layer_norm_out(xr[i] - mu, denom, i, weight, bias, o);
         }
     }
 }
+
+// smallest register-resident variant that holds a row of n values, 0 for the streaming one
+int row_chunks(long n)
+{
+    for (int ch : {1, 2, 4, 8, 16}) if (n <= 64L * ch) return ch;
+    return 0;
+}
+
+#define PAM_ROW_DISPATCH(KERNEL, n, grid, st, ...)                                                              \
+    switch (row_chunks(n)) {                                                                                    \
+    case 1: hipLaunchKernelGGL(KERNEL<1>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 2: hipLaunchKernelGGL(KERNEL<2>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 4: hipLaunchKernelGGL(KERNEL<4>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 16: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
+    default: hipLaunchKernelGGL(KERNEL<0>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                    \
+    }
 
 int g_cus = 0;
 int cu_count()
@@ -261,11 +378,13 @@ int launch_max(const char* what, const float* x, long rows, long n, Offset o, in
     if (!workspace || workspace_bytes < pam_hip_rowop_workspace_bytes())
         return pamhost::fail(PAM_HIP_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", what, pam_hip_rowop_workspace_bytes());
     size_t total = (size_t)rows * (size_t)n;
+    size_t nvec = ((uintptr_t)x & 15u) ? 0 : total / 4;
     size_t blocks = (total + (size_t)kThreads * 16 - 1) / ((size_t)kThreads * 16);
     if (blocks > (size_t)kMaxPartials) blocks = kMaxPartials;
     if (blocks < 1) blocks = 1;
     *partials = (int)blocks;
-    hipLaunchKernelGGL(scaled_max_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, x, total, o, mask_inf, (float*)workspace);
+    hipLaunchKernelGGL(scaled_max_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, x, total, nvec, o, mask_inf,
+                       (float*)workspace);
     return pamhost::check_launch(what);
 }
 
@@ -285,8 +404,8 @@ int pam_hip_softmax_fwd(const float* x, float* y, float* row_sum, float* shift, 
     hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
     rc = launch_max("softmax_fwd", x, rows, n, o, 1, workspace, workspace_bytes, st, &partials);
     if (rc != PAM_HIP_OK) return rc;
-    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, st, x, y, row_sum, shift, rows, n, o,
-                       (const float*)workspace, partials);
+    PAM_ROW_DISPATCH(softmax_fwd_kernel, n, dim3(row_grid(rows)), st, x, y, row_sum, shift, rows, n, o,
+                     (const float*)workspace, partials);
     return pamhost::check_launch("softmax_fwd");
 }
 
@@ -298,8 +417,7 @@ int pam_hip_softmax_bwd(const float* x, const float* dy, const float* row_sum, c
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !dy || !row_sum || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "softmax_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    hipLaunchKernelGGL(softmax_bwd_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream,
-                       x, dy, row_sum, shift, dx, rows, n, o, ap);
+    PAM_ROW_DISPATCH(softmax_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap);
     return pamhost::check_launch("softmax_bwd");
 }
 
@@ -313,8 +431,8 @@ int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, long r
     hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
     rc = launch_max("logsumexp_fwd", x, rows, n, o, 0, workspace, workspace_bytes, st, &partials);
     if (rc != PAM_HIP_OK) return rc;
-    hipLaunchKernelGGL(logsumexp_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, st, x, lse, log_softmax, rows, n, o,
-                       (const float*)workspace, partials);
+    PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows)), st, x, lse, log_softmax, rows, n, o,
+                     (const float*)workspace, partials);
     return pamhost::check_launch("logsumexp_fwd");
 }
 
@@ -336,8 +454,8 @@ int pam_hip_layer_norm_fwd(const float* x, const float* weight, const float* bia
     if (rc != PAM_HIP_OK) return rc;
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !y) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_fwd: null pointer");
-    hipLaunchKernelGGL(layer_norm_fwd_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, weight, bias, y,
-                       rows, n, eps, Offset{offset, offset != 1.0f});
+    const Offset o{offset, offset != 1.0f};
+    PAM_ROW_DISPATCH(layer_norm_fwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, bias, y, rows, n, eps, o);
     return pamhost::check_launch("layer_norm_fwd");
 }
 
