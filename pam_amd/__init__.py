@@ -8,6 +8,8 @@ The names of the reference's `pam` package that live on this path are re-exporte
 """
 from .pam_ops import *          # noqa: F401,F403
 from .composites import *       # noqa: F401,F403
+from .pam_opt import *          # noqa: F401,F403
+from . import pam_experimental  # noqa: F401
 from . import cuda_bindings     # noqa: F401
 from . import pam_ops           # noqa: F401
 from . import composites        # noqa: F401
