@@ -145,6 +145,18 @@ int pam_hip_row_mean_fwd(const float *x, float *y, long rows, long n, float offs
 int pam_hip_layer_norm_fwd(const float *x, const float *weight, const float *bias, float *y, long rows, long n,
                            float eps, float offset, void *stream);
 
+/* ---- optimizer step ---------------------------------------------------------------------- */
+/* One Adam update of n parameters in place, every product, the quotient and the square root
+ * a PAM op                replaces the op-table arithmetic of the training recipe's optimizer
+ * (submodules/fairseq/fairseq/optim/adam.py:226-252 in the reference tree):
+ *   m = m (*) beta1 + g (*) (1 - beta1);   v = v (*) beta2;   v += (g (*) g) (*) (1 - beta2)
+ *   denom = pow(v, 0.5) + eps;   if has_decay: p -= p (*) decay;   p -= (m (/) denom) (*) step_size
+ * The scalars are the fp32 roundings of the host's double-precision values (decay = weight
+ * decay x learning rate, step_size = lr sqrt(1 - beta2^t) / (1 - beta1^t)). */
+int pam_hip_adam_step(float *p, const float *g, float *m, float *v, size_t n, float beta1, float one_minus_beta1,
+                      float beta2, float one_minus_beta2, float eps, float decay, int has_decay, float step_size,
+                      float offset, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

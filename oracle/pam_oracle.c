@@ -551,4 +551,23 @@ void pamo_layer_norm_fwd(const float *x, const float *weight, const float *bias,
     }
 }
 
+/* One Adam update with PAM ops (submodules/fairseq/fairseq/optim/adam.py:226-252 of the
+ * reference tree), the chain of primitive calls written out; in place. */
+void pamo_adam_step(float *p, const float *g, float *m, float *v, size_t n, float beta1, float one_minus_beta1,
+                    float beta2, float one_minus_beta2, float eps, float decay, int has_decay, float step_size, float off)
+{
+    #pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        volatile float m1 = pam_off(m[i], beta1, off) + pam_off(g[i], one_minus_beta1, off);
+        volatile float v0 = pam_off(v[i], beta2, off);
+        volatile float v1 = v0 + pam_off(pam_off(g[i], g[i], off), one_minus_beta2, off);
+        float root = v1 == 0.0f ? 0.0f : exp2_op(pam_off(log2_op(v1, off), 0.5f, off), off);
+        volatile float denom = root + eps;
+        volatile float p1 = p[i];
+        if (has_decay) p1 = p1 - pam_off(p1, decay, off);
+        volatile float p2 = p1 - pam_off(pad_off(m1, denom, off), step_size, off);
+        p[i] = p2; m[i] = m1; v[i] = v1;
+    }
+}
+
 int pamo_version(void) { return 2; }

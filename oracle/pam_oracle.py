@@ -63,6 +63,8 @@ def lib():
         L.pamo_logsumexp_fwd.argtypes = [_fp, _fp, _fp, cl, cl, cf]
         L.pamo_row_mean_fwd.argtypes = [_fp, _fp, cl, cl, cf]
         L.pamo_layer_norm_fwd.argtypes = [_fp, _fp, _fp, _fp, cl, cl, cf, cf]
+        L.pamo_adam_step.argtypes = [_fp, _fp, _fp, _fp, ctypes.c_size_t, cf, cf, cf, cf, cf, cf, ci, cf, cf]
+        L.pamo_adam_step.restype = None
         for name in ("pamo_softmax_fwd", "pamo_softmax_bwd", "pamo_logsumexp_fwd", "pamo_row_mean_fwd",
                      "pamo_layer_norm_fwd"):
             getattr(L, name).restype = None
@@ -258,3 +260,12 @@ def layer_norm_fwd(x, weight=None, bias=None, eps=1e-5, offset=None):
     lib().pamo_layer_norm_fwd(_p(x2), None if w is None else _p(w), None if b is None else _p(b), _p(y),
                               x2.shape[0], x2.shape[1], float(np.float32(eps)), _off(offset))
     return y.reshape(shape)
+
+
+def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, decay, step_size, offset=None):
+    """Returns the updated (p, m, v); decay None or 0 skips the weight-decay term."""
+    p, g, m, v = (_f32(t).copy() for t in (p, g, m, v))
+    f = lambda x: float(np.float32(x))
+    lib().pamo_adam_step(_p(p), _p(g), _p(m), _p(v), p.size, f(beta1), f(one_minus_beta1), f(beta2), f(one_minus_beta2),
+                         f(eps), f(decay or 0.0), int(bool(decay)), f(step_size), _off(offset))
+    return p, m, v

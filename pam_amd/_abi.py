@@ -43,6 +43,7 @@ _SIGNATURES = {
     "pam_hip_standard_bmm": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_matmul_bwd": (_MAT2 * 4 + [_l, _l, _l, _i, _f, _p, _z, _p], _i),
     "pam_hip_pam_bmm_bwd": (_MAT * 4 + [_l, _l, _l, _l, _i, _f, _p, _z, _p], _i),
+    "pam_hip_adam_step": ([_p, _p, _p, _p, _z, _f, _f, _f, _f, _f, _f, _i, _f, _f, _p], _i),
     "pam_hip_rowop_workspace_bytes": ([], _z),
     "pam_hip_softmax_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_softmax_bwd": ([_p, _p, _p, _p, _p, _l, _l, _f, _i, _i, _i, _p], _i),
@@ -334,3 +335,18 @@ class HipRowKernels:
                 _call("pam_hip_layer_norm_fwd", X.data_ptr(), None if weight is None else weight.data_ptr(),
                       None if bias is None else bias.data_ptr(), Y.data_ptr(), rows, n, float(eps), float(offset), _stream())
         return Y
+
+
+def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, decay, step_size, offset):
+    """In-place Adam update of the contiguous fp32 GPU tensors p, m, v from the gradient g;
+    decay None or 0 skips the weight-decay term."""
+    _check(p, g, m, v)
+    if not (p.is_contiguous() and g.is_contiguous() and m.is_contiguous() and v.is_contiguous()):
+        raise ValueError("adam_step: tensors must be contiguous")
+    if not (p.shape == g.shape == m.shape == v.shape):
+        raise ValueError("adam_step: tensors must have the same shape")
+    if p.numel():
+        with torch.cuda.device(p.device):
+            _call("pam_hip_adam_step", p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), float(beta1),
+                  float(one_minus_beta1), float(beta2), float(one_minus_beta2), float(eps), float(decay or 0.0),
+                  int(bool(decay)), float(step_size), float(offset), _stream())

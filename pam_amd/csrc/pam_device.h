@@ -218,4 +218,15 @@ __device__ __forceinline__ float pa_log2_signed(float x)
     return pa_log2(x);
 }
 
+// exp2, log2 and the square root as the op library reaches them: through the base-2 forms of
+// the exp / log entry points, pa_exp2(t (*) log2 2) and pa_log2(v) (/) log2 2
+// (pam/cuda_bindings.py:246, 283), and pow(v, 0.5) = exp2(log2(v) (*) 0.5) with zero kept at
+// zero (pam/pam_ops.py:70-79).
+__device__ __forceinline__ float exp2_entry(float t, float off, bool has_off)
+{ return pa_exp2(pam_mul_off(t, 1.0f, off, has_off)); }
+__device__ __forceinline__ float log2_entry(float v, float off, bool has_off)
+{ return pad_div_off(pa_log2(v), 1.0f, off, has_off); }
+__device__ __forceinline__ float pow_half(float v, float off, bool has_off)
+{ return v == 0.0f ? 0.0f : exp2_entry(pam_mul_off(log2_entry(v, off, has_off), 0.5f, off, has_off), off, has_off); }
+
 }  // namespace pamdev

@@ -135,6 +135,55 @@ int launch(const char* what, const float* p0, const float* p1, const float* p2, 
     return pamhost::check_launch(what);
 }
 
+// ---------------------------------------------------------------- Adam step
+// One update of a parameter tensor by the Adam variant whose products, quotient and square
+// root are PAM ops (the training recipe's optimizer, fairseq/optim/adam.py:226-252 in the
+// reference tree): eleven elementwise launches there, one here.  Reads p, g, m, v and
+// writes p, m, v: 28 B/element.
+struct AdamArgs {
+    float beta1, one_minus_beta1, beta2, one_minus_beta2, eps, decay, step_size, off;
+    bool has_decay, has_off;
+};
+
+__device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, const AdamArgs& a)
+{
+    const float off = a.off; const bool ho = a.has_off;
+    m = pam_mul_off(m, a.beta1, off, ho) + pam_mul_off(g, a.one_minus_beta1, off, ho);
+    v = pam_mul_off(v, a.beta2, off, ho);
+    v = v + pam_mul_off(pam_mul_off(g, g, off, ho), a.one_minus_beta2, off, ho);
+    const float denom = pow_half(v, off, ho) + a.eps;
+    if (a.has_decay) p = p - pam_mul_off(p, a.decay, off, ho);
+    p = p - pam_mul_off(pad_div_off(m, denom, off, ho), a.step_size, off, ho);
+}
+
+__global__ __launch_bounds__(kThreads) void adam_vec_kernel(v4f* __restrict__ p, const v4f* __restrict__ g,
+                                                           v4f* __restrict__ m, v4f* __restrict__ v, size_t nvec, AdamArgs a)
+{
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += step) {
+        v4f pp = p[i], gg = __builtin_nontemporal_load(g + i), mm = m[i], vv = v[i];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            float pc = pp[c], mc = mm[c], vc = vv[c];
+            adam_one(pc, gg[c], mc, vc, a);
+            pp[c] = pc; mm[c] = mc; vv[c] = vc;
+        }
+        p[i] = pp; m[i] = mm; v[i] = vv;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void adam_scalar_kernel(float* __restrict__ p, const float* __restrict__ g,
+                                                              float* __restrict__ m, float* __restrict__ v,
+                                                              size_t first, size_t n, AdamArgs a)
+{
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (size_t i = first + (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += step) {
+        float pp = p[i], mm = m[i], vv = v[i];
+        adam_one(pp, g[i], mm, vv, a);
+        p[i] = pp; m[i] = mm; v[i] = vv;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -194,5 +243,30 @@ int pam_hip_pa_exp_bwd(const float* x, const float* dy, float* dx, size_t n, flo
 
 int pam_hip_pa_log_bwd(const float* x, const float* dy, float* dx, size_t n, float base, float offset, void* stream)
 { return launch<OpLogBwd, 2>("pa_log_bwd", x, dy, nullptr, dx, n, OpLogBwd{log2f(base), offset, offset != 1.0f}, stream); }
+
+int pam_hip_adam_step(float* p, const float* g, float* m, float* v, size_t n, float beta1, float one_minus_beta1,
+                      float beta2, float one_minus_beta2, float eps, float decay, int has_decay, float step_size,
+                      float offset, void* stream)
+{
+    if (n == 0) return PAM_HIP_OK;
+    if (!p || !g || !m || !v) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "adam_step: null pointer");
+    AdamArgs a{beta1, one_minus_beta1, beta2, one_minus_beta2, eps, decay, step_size, offset, has_decay != 0, offset != 1.0f};
+    hipStream_t st = (hipStream_t)stream;
+    uintptr_t align = (uintptr_t)p | (uintptr_t)g | (uintptr_t)m | (uintptr_t)v;
+    size_t nvec = (align & 15u) ? 0 : n / 4;
+    const size_t cap = (size_t)1 << 30;
+    if (nvec) {
+        size_t blocks = (nvec + kThreads - 1) / kThreads;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(adam_vec_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, (v4f*)p, (const v4f*)g, (v4f*)m,
+                           (v4f*)v, nvec, a);
+    }
+    if (nvec * 4 < n) {
+        size_t blocks = (n - nvec * 4 + kThreads - 1) / kThreads;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(adam_scalar_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, p, g, m, v, nvec * 4, n, a);
+    }
+    return pamhost::check_launch("adam_step");
+}
 
 }  // extern "C"

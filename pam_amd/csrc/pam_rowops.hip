@@ -58,9 +58,9 @@ __device__ __forceinline__ float scaled(float x, Offset o, bool mask_inf)
 }
 
 // exp2 through the kernel entry point of that name: pa_exp2(t (*) log2(2)) (pam/cuda_bindings.py:246)
-__device__ __forceinline__ float exp2_op(float t, Offset o) { return pa_exp2(pam_mul_off(t, 1.0f, o.off, o.has)); }
+__device__ __forceinline__ float exp2_op(float t, Offset o) { return exp2_entry(t, o.off, o.has); }
 // log2 likewise: pa_log2(v) (/) log2(2)
-__device__ __forceinline__ float log2_op(float v, Offset o) { return pad_div_off(pa_log2(v), 1.0f, o.off, o.has); }
+__device__ __forceinline__ float log2_op(float v, Offset o) { return log2_entry(v, o.off, o.has); }
 
 // ---------------------------------------------------------------- global maximum of the scaled input
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -283,8 +283,7 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restr
 
 // ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
 // pow(v, 0.5) = exp2(log2(v) (*) 0.5), zero at zero (pam/pam_ops.py:70-79)
-__device__ __forceinline__ float root_op(float v, Offset o)
-{ return v == 0.0f ? 0.0f : exp2_op(pam_mul_off(log2_op(v, o), 0.5f, o.off, o.has), o); }
+__device__ __forceinline__ float root_op(float v, Offset o) { return pow_half(v, o.off, o.has); }
 
 __device__ __forceinline__ float layer_norm_out(float centred, float denom, long i, const float* __restrict__ weight,
                                                const float* __restrict__ bias, Offset o)
