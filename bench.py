@@ -180,6 +180,33 @@ def main():
         for name, (ops, macs, fn) in exact.items():
             ms = event_time_ms(fn, 10, torch)
             other[name] = {"ms": round(ms, 4), "gmacs": round(macs / ms / 1e6, 1), "valu_frac": round(ops * macs / (ms * 1e-3) / lane_peak, 4)}
+        # row-wise compositions as single kernels and the Adam step (HBM-bound; algorithmic bytes per element)
+        from pam_amd import _abi as abi
+        R = abi.HipRowKernels()
+        rows_cases = {"attention_37824x197": (192 * 197, 197), "rows_65536x1024": (65536, 1024)}
+        for tag, (r, c) in rows_cases.items():
+            xs = torch.randn(r, c, generator=g).to(dev); gs = torch.randn(r, c, generator=g).to(dev)
+            wv = torch.randn(c, generator=g).to(dev); bv = torch.randn(c, generator=g).to(dev)
+            ys, rs, sh = R.softmax_fwd(xs, 1.0)
+            row_ops = (
+                ("softmax_fwd", 12, lambda: R.softmax_fwd(xs, 1.0)),
+                ("softmax_bwd_approx", 12, lambda: R.softmax_bwd(xs, gs, rs, sh, 1.0, True, True, True)),
+                ("softmax_bwd_exact", 12, lambda: R.softmax_bwd(xs, gs, rs, sh, 1.0, False, False, False)),
+                ("log_softmax_fwd", 12, lambda: R.logsumexp_fwd(xs, 1.0, False, True)),
+                ("layer_norm_fwd", 8, lambda: R.layer_norm_fwd(xs, wv, bv, 1e-5, 1.0)),
+                ("row_mean_fwd", 4, lambda: R.row_mean_fwd(xs, 1.0)),
+            )
+            for name, bpe, fn in row_ops:
+                ms = event_time_ms(fn, 10, torch)
+                other[f"{name}_{tag}"] = {"ms": round(ms, 4), "GBps": round(bpe * r * c / ms / 1e6, 1),
+                                          "hbm_frac": round(bpe * r * c / ms / 1e6 / 8000.0, 3)}
+            del xs, gs, ys
+        na = 1 << 26
+        pa, ga, ma, va = (torch.randn(na, generator=g).to(dev) * s_ for s_ in (1.0, 1e-2, 1e-2, 1e-4))
+        va.abs_()
+        ms = event_time_ms(lambda: abi.adam_step(pa, ga, ma, va, 0.9, 0.1, 0.98, 0.02, 1e-8, 5e-8, 4e-4, 1.0), 10, torch)
+        other["adam_step_2p26"] = {"ms": round(ms, 4), "GBps": round(28 * na / ms / 1e6, 1), "hbm_frac": round(28 * na / ms / 1e6 / 8000.0, 3)}
+        del pa, ga, ma, va
         out["other_kernels"] = other
 
     if not args.no_cpu_baseline:
