@@ -229,4 +229,59 @@ __device__ __forceinline__ float log2_entry(float v, float off, bool has_off)
 __device__ __forceinline__ float pow_half(float v, float off, bool has_off)
 { return v == 0.0f ? 0.0f : exp2_entry(pam_mul_off(log2_entry(v, off, has_off), 0.5f, off, has_off), off, has_off); }
 
+// ---------------------------------------------------------------- unchecked forms
+// Chains of many primitive calls per element (row kernels, optimizer step) pay a range check
+// and a branch per call when built from the functions above.  The forms below compute the
+// normal-range result without branching and fold every magnitude they touch into a running
+// min / max; `Span::normal()` then tells, once per chain, whether each operand and each
+// result was a normal number -- in which case every value equals what the checked function
+// returns -- or the chain has to be redone with the checked functions.
+struct Span {
+    uint32_t lo = 0x7f7fffffu, hi = 0x00800000u;
+    bool in_exp_range = true;
+    __device__ __forceinline__ void see(uint32_t mag) { lo = min(lo, mag); hi = max(hi, mag); }
+    __device__ __forceinline__ bool normal() const { return in_exp_range && lo >= 0x00800000u && hi < kExpo; }
+};
+
+__device__ __forceinline__ float pam_unchecked(float a, float b, Span& sp)
+{
+    uint32_t ai = f2u(a), bi = f2u(b), ma = ai & ~kSign, mb = bi & ~kSign;
+    uint32_t s = ma + mb - kBias;
+    sp.see(ma); sp.see(mb); sp.see(s);
+    return u2f(s | ((ai ^ bi) & kSign));
+}
+__device__ __forceinline__ float pad_unchecked(float a, float b, Span& sp)
+{
+    uint32_t ai = f2u(a), bi = f2u(b), ma = ai & ~kSign, mb = bi & ~kSign;
+    uint32_t s = ma - mb + kBias;                 // a wrap lands above the exponent mask and is caught
+    sp.see(ma); sp.see(mb); sp.see(s);
+    return u2f(s | ((ai ^ bi) & kSign));
+}
+__device__ __forceinline__ float pam_unchecked_off(float a, float b, float off, bool has_off, Span& sp)
+{ float c = pam_unchecked(a, b, sp); return has_off ? pam_unchecked(c, off, sp) : c; }
+__device__ __forceinline__ float pad_unchecked_off(float a, float b, float off, bool has_off, Span& sp)
+{ float c = pad_unchecked(a, b, sp); return has_off ? pad_unchecked(c, off, sp) : c; }
+
+// pa_log2 of a normal number: (bits(|x|) - bias) / 2^23, one rounding in the conversion
+__device__ __forceinline__ float pa_log2_unchecked(float x, Span& sp)
+{
+    uint32_t mag = f2u(x) & ~kSign;
+    sp.see(mag);
+    return (float)((int)mag - (int)kBias) * 0x1p-23f;
+}
+// pa_exp2 for -126 <= floor(x) <= 127, where 2**floor(x) is a normal number
+__device__ __forceinline__ float pa_exp2_unchecked(float x, Span& sp)
+{
+    sp.in_exp_range = sp.in_exp_range && (x >= -126.0f) && (x < 128.0f);       // false for NaN
+    float f = floorf(x);
+    float t = (1.0f + x) - f;
+    return u2f((uint32_t)((int)f + 127) << 23) * t;
+}
+__device__ __forceinline__ float exp2_entry_unchecked(float t, float off, bool has_off, Span& sp)
+{ return pa_exp2_unchecked(pam_unchecked_off(t, 1.0f, off, has_off, sp), sp); }
+__device__ __forceinline__ float log2_entry_unchecked(float v, float off, bool has_off, Span& sp)
+{ return pad_unchecked_off(pa_log2_unchecked(v, sp), 1.0f, off, has_off, sp); }
+__device__ __forceinline__ float pow_half_unchecked(float v, float off, bool has_off, Span& sp)
+{ return exp2_entry_unchecked(pam_unchecked_off(log2_entry_unchecked(v, off, has_off, sp), 0.5f, off, has_off, sp), off, has_off, sp); }
+
 }  // namespace pamdev

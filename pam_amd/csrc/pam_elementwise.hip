@@ -145,6 +145,18 @@ struct AdamArgs {
     bool has_decay, has_off;
 };
 
+// the update with every operand and result in the normal range: no branches; `sp` records whether that held
+__device__ __forceinline__ void adam_one_unchecked(float& p, float g, float& m, float& v, const AdamArgs& a, Span& sp)
+{
+    const float off = a.off; const bool ho = a.has_off;
+    m = pam_unchecked_off(m, a.beta1, off, ho, sp) + pam_unchecked_off(g, a.one_minus_beta1, off, ho, sp);
+    v = pam_unchecked_off(v, a.beta2, off, ho, sp);
+    v = v + pam_unchecked_off(pam_unchecked_off(g, g, off, ho, sp), a.one_minus_beta2, off, ho, sp);
+    const float denom = pow_half_unchecked(v, off, ho, sp) + a.eps;
+    if (a.has_decay) p = p - pam_unchecked_off(p, a.decay, off, ho, sp);
+    p = p - pam_unchecked_off(pad_unchecked_off(m, denom, off, ho, sp), a.step_size, off, ho, sp);
+}
+
 __device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, const AdamArgs& a)
 {
     const float off = a.off; const bool ho = a.has_off;
@@ -162,13 +174,23 @@ __global__ __launch_bounds__(kThreads) void adam_vec_kernel(v4f* __restrict__ p,
     const size_t step = (size_t)gridDim.x * kThreads;
     for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += step) {
         v4f pp = p[i], gg = __builtin_nontemporal_load(g + i), mm = m[i], vv = v[i];
+        v4f p1 = pp, m1 = mm, v1 = vv;
+        Span sp;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             float pc = pp[c], mc = mm[c], vc = vv[c];
-            adam_one(pc, gg[c], mc, vc, a);
-            pp[c] = pc; mm[c] = mc; vv[c] = vc;
+            adam_one_unchecked(pc, gg[c], mc, vc, a, sp);
+            p1[c] = pc; m1[c] = mc; v1[c] = vc;
         }
-        p[i] = pp; m[i] = mm; v[i] = vv;
+        if (!sp.normal()) {                     // a zero, subnormal, inf, NaN or out-of-range value somewhere: redo checked
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float pc = pp[c], mc = mm[c], vc = vv[c];
+                adam_one(pc, gg[c], mc, vc, a);
+                p1[c] = pc; m1[c] = mc; v1[c] = vc;
+            }
+        }
+        p[i] = p1; m[i] = m1; v[i] = v1;
     }
 }
 

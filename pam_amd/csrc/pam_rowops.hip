@@ -22,6 +22,9 @@ using namespace pamdev;
 
 namespace {
 
+#ifndef PAM_ROW_WAVES
+#define PAM_ROW_WAVES 4
+#endif
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 constexpr int kMaxPartials = 1024;
@@ -135,6 +138,35 @@ __device__ __forceinline__ float stream_sum(const float* __restrict__ p, long n,
     return acc;
 }
 
+// ---------------------------------------------------------------- checked and unchecked arithmetic
+// A register-resident row is first computed with the unchecked forms of the primitives (no
+// branches; they record whether every operand and result was a normal number).  If any lane of
+// the wavefront saw anything else -- a zero, a subnormal, inf, NaN, an exponent out of range --
+// the row is redone with the checked functions.  Both give the same bits whenever the first
+// is valid, so which one ran never shows in the result.
+struct Checked {
+    Offset o;
+    __device__ __forceinline__ float mul(float a, float b) { return pam_mul_off(a, b, o.off, o.has); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_div_off(a, b, o.off, o.has); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry(t, o.off, o.has); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry(v, o.off, o.has); }
+    __device__ __forceinline__ float root(float v) { return pow_half(v, o.off, o.has); }
+    // 0 (/) b for an element whose weight is exactly zero
+    __device__ __forceinline__ float zero_over(float b) { return pad_div_off(0.0f, b, o.off, o.has); }
+    __device__ __forceinline__ bool valid() const { return true; }
+};
+struct Unchecked {
+    Offset o; Span sp;
+    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, o.has, sp); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, o.has, sp); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, o.has, sp); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float root(float v) { return pow_half_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float zero_over(float) { return 0.0f; }      // the divisor is a positive normal number when valid
+    __device__ __forceinline__ bool valid() const { return sp.normal(); }
+};
+__device__ __forceinline__ bool wave_valid(const Unchecked& u) { return __ballot(!u.valid()) == 0ull; }
+
 // ---------------------------------------------------------------- softmax forward (pam/pam_ops.py:305-328)
 __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
 {
@@ -142,8 +174,31 @@ __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
     return exp2_op(scaled(x, o, false) - shift, o);
 }
 
+// one row held in registers: weights, their sum, the quotients; masked (-inf) elements weigh exactly zero
+template <int CH, class M>
+__device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)[CH], float shift, M& m)
+{
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool masked = f2u(xv[c]) == 0xff800000u;       // computed on stand-in values, then replaced
+        const float t = m.mul(masked ? 1.0f : xv[c], kLog2E) - shift;
+        const float e = m.exp2(masked ? 0.5f : t);
+        out[c] = masked ? 0.0f : e;
+        p = p + out[c];
+    }
+    const float total = wave_sum(p);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool masked = f2u(xv[c]) == 0xff800000u;
+        const float q = m.div(masked ? 1.0f : out[c], total);
+        out[c] = masked ? m.zero_over(total) : q;
+    }
+    return total;
+}
+
 template <int CH>
-__global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                               float* __restrict__ row_sum, float* __restrict__ shift_out,
                                                               long rows, long n, Offset o,
                                                               const float* __restrict__ partial, int partials)
@@ -156,14 +211,13 @@ __global__ __launch_bounds__(kThreads) void softmax_fwd_kernel(const float* __re
         const float* xr = x + r * n; float* yr = y + r * n;
         float total;
         if constexpr (CH > 0) {
-            float e[CH];
-            load_row<CH>(e, xr, n, lane, kNegInf);             // the fill has weight zero
-            float p = 0.0f;
+            float xv[CH], out[CH];
+            load_row<CH>(xv, xr, n, lane, kNegInf);            // the fill has weight zero
+            Unchecked u{o};
+            total = softmax_row<CH>(xv, out, shift, u);
+            if (!wave_valid(u)) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k); }
 #pragma unroll
-            for (int c = 0; c < CH; ++c) { e[c] = softmax_weight(e[c], shift, o); p = p + e[c]; }
-            total = wave_sum(p);
-#pragma unroll
-            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = pad_div_off(e[c], total, o.off, o.has); }
+            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
             total = wave_sum(stream_sum(xr, n, lane, [&](long, float v) { return softmax_weight(v, shift, o); }));
             for (long i = lane; i < n; i += 64) yr[i] = pad_div_off(softmax_weight(xr[i], shift, o), total, o.off, o.has);
@@ -197,8 +251,42 @@ __device__ __forceinline__ float softmax_dx(float xv, float e, float g, float in
     return ap.a ? pam_mul_off(dt, kLog2E, o.off, o.has) : pam_mul_bwd(xv, kLog2E, dt, o.off, o.has);
 }
 
+// The all-approximate gradient of one register-resident row with unchecked arithmetic.  Masked
+// (-inf) elements and the lanes past the end of the row are computed on a stand-in value and
+// replaced by the zeros the chain gives them.
 template <int CH>
-__global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+__device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
+                                                        float total, float shift, int lane, long n, Unchecked& m)
+{
+    const float inv = m.div(1.0f, total);
+    float e[CH];
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool masked = f2u(xv[c]) == 0xff800000u;
+        const bool inside = lane + 64L * c < n;
+        const float t = m.mul(masked ? 1.0f : xv[c], kLog2E) - shift;
+        e[c] = m.exp2(masked ? 0.5f : t);                                  // exp2 of the shifted input, unmasked
+        // -(((e (/) total) (/) total) (*) g); a masked element has e = 0 and the checked chain gives
+        // -(0 (*) g), a zero for finite g (adding it changes nothing: the sum is never -0) and NaN otherwise
+        const float term = -m.mul(m.div(m.div(e[c], total), total), (inside && !masked) ? g[c] : 1.0f);
+        if (masked && inside) m.sp.see(f2u(g[c]) & ~kSign);
+        if (inside && !masked) p = p + term;
+    }
+    const float dtotal = wave_sum(p);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool masked = f2u(xv[c]) == 0xff800000u;
+        const bool inside = lane + 64L * c < n;
+        const float de = m.mul(inv, (inside && !masked) ? g[c] : 1.0f) + dtotal;
+        const float dt = m.mul(m.mul(e[c], kLn2), de);
+        const float dx = m.mul(dt, kLog2E);
+        out[c] = masked ? 0.0f : dx;
+    }
+}
+
+template <int CH>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                               const float* __restrict__ row_sum, const float* __restrict__ shift_in,
                                                               float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
 {
@@ -210,21 +298,29 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const float* __re
         const float total = row_sum[r];
         const float inv = pad_div_off(1.0f, total, o.off, o.has);
         if constexpr (CH > 0) {
-            float xv[CH], g[CH], e[CH];
+            float xv[CH], g[CH], out[CH];
             load_row<CH>(xv, xr, n, lane, kNegInf);
             load_row<CH>(g, gr, n, lane, 0.0f);
-            float p = 0.0f;
-#pragma unroll
-            for (int c = 0; c < CH; ++c) {
-                e[c] = softmax_weight(xv[c], shift, o);
-                if (lane + 64L * c < n) p = p + softmax_dsum_term(e[c], total, g[c], o, ap);
+            bool done = false;
+            if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient has an unchecked form
+                Unchecked u{o};
+                softmax_grad_row_approx<CH>(xv, g, out, total, shift, lane, n, u);
+                done = wave_valid(u);
             }
-            const float dtotal = wave_sum(p);
+            if (!done) {
+                float e[CH];
+                float p = 0.0f;
 #pragma unroll
-            for (int c = 0; c < CH; ++c) {
-                long i = lane + 64L * c;
-                if (i < n) dr[i] = softmax_dx(xv[c], e[c], g[c], inv, dtotal, shift, o, ap);
+                for (int c = 0; c < CH; ++c) {
+                    e[c] = softmax_weight(xv[c], shift, o);
+                    if (lane + 64L * c < n) p = p + softmax_dsum_term(e[c], total, g[c], o, ap);
+                }
+                const float dtotal = wave_sum(p);
+#pragma unroll
+                for (int c = 0; c < CH; ++c) out[c] = softmax_dx(xv[c], e[c], g[c], inv, dtotal, shift, o, ap);
             }
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) dr[i] = out[c]; }
         } else {
             const float dtotal = wave_sum(stream_sum(xr, n, lane, [&](long i, float v) {
                 return softmax_dsum_term(softmax_weight(v, shift, o), total, gr[i], o, ap); }));
@@ -237,8 +333,22 @@ __global__ __launch_bounds__(kThreads) void softmax_bwd_kernel(const float* __re
 }
 
 // ---------------------------------------------------------------- logsumexp and log_softmax (pam/pam_ops.py:331-347)
+template <int CH, class M>
+__device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shift, int lane, long n, M& m)
+{
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool inside = lane + 64L * c < n;                  // lanes past the end work on stand-in values
+        const float t = m.mul(inside ? xv[c] : 1.0f, kLog2E) - shift;
+        const float e = m.exp2(inside ? t : 0.5f);
+        if (inside) p = p + e;
+    }
+    return m.div(shift + m.log2(wave_sum(p)), kLog2E);
+}
+
 template <int CH>
-__global__ __launch_bounds__(kThreads) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
                                                             float* __restrict__ y, long rows, long n, Offset o,
                                                             const float* __restrict__ partial, int partials)
 {
@@ -251,10 +361,9 @@ __global__ __launch_bounds__(kThreads) void logsumexp_kernel(const float* __rest
         if constexpr (CH > 0) {
             float xv[CH];
             load_row<CH>(xv, xr, n, lane, 0.0f);
-            float p = 0.0f;
-#pragma unroll
-            for (int c = 0; c < CH; ++c) if (lane + 64L * c < n) p = p + weight(0, xv[c]);
-            const float out = pad_div_off(shift + log2_op(wave_sum(p), o), kLog2E, o.off, o.has);
+            Unchecked u{o};
+            float out = logsumexp_row<CH>(xv, shift, lane, n, u);
+            if (!wave_valid(u)) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lane, n, k); }
             if (lse && lane == 0) lse[r] = out;
             if (y) {
 #pragma unroll
@@ -294,8 +403,34 @@ __device__ __forceinline__ float layer_norm_out(float centred, float denom, long
     return out;
 }
 
+template <int CH, class M>
+__device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&out)[CH], const float* __restrict__ weight,
+                                               const float* __restrict__ bias, int lane, long n, float count, float eps, M& m)
+{
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) p = p + xv[c];                          // the fill adds +0
+    const float mu = m.div(wave_sum(p), count);
+    p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        out[c] = xv[c] - mu;                                             // lanes past the end hold -mu, a stand-in
+        const float sq = m.mul(out[c], out[c]);
+        if (lane + 64L * c < n) p = p + sq;
+    }
+    const float denom = m.root(m.div(wave_sum(p), count) + eps);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const long i = lane + 64L * c; const bool inside = i < n;
+        float r = m.div(out[c], denom);
+        if (weight) r = m.mul(r, inside ? weight[i] : 1.0f);
+        if (bias) r = r + (inside ? bias[i] : 0.0f);
+        out[c] = r;
+    }
+}
+
 template <int CH>
-__global__ __launch_bounds__(kThreads) void layer_norm_fwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void layer_norm_fwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
                                                                  const float* __restrict__ bias, float* __restrict__ y,
                                                                  long rows, long n, float eps, Offset o)
 {
@@ -305,18 +440,13 @@ __global__ __launch_bounds__(kThreads) void layer_norm_fwd_kernel(const float* _
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
         if constexpr (CH > 0) {
-            float v[CH];
-            load_row<CH>(v, xr, n, lane, 0.0f);
-            float p = 0.0f;
+            float xv[CH], out[CH];
+            load_row<CH>(xv, xr, n, lane, 0.0f);
+            Unchecked u{o};
+            layer_norm_row<CH>(xv, out, weight, bias, lane, n, count, eps, u);
+            if (!wave_valid(u)) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lane, n, count, eps, k); }
 #pragma unroll
-            for (int c = 0; c < CH; ++c) p = p + v[c];                       // the fill adds +0
-            const float mu = pad_div_off(wave_sum(p), count, o.off, o.has);
-            p = 0.0f;
-#pragma unroll
-            for (int c = 0; c < CH; ++c) { v[c] = v[c] - mu; if (lane + 64L * c < n) p = p + pam_mul_off(v[c], v[c], o.off, o.has); }
-            const float denom = root_op(pad_div_off(wave_sum(p), count, o.off, o.has) + eps, o);
-#pragma unroll
-            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = layer_norm_out(v[c], denom, i, weight, bias, o); }
+            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
             const float mu = pad_div_off(wave_sum(stream_sum(xr, n, lane, [](long, float v) { return v; })), count, o.off, o.has);
             const float var = pad_div_off(wave_sum(stream_sum(xr, n, lane, [&](long, float v) {
