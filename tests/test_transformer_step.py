@@ -10,6 +10,17 @@ import pam_amd
 from pam_amd import cuda_bindings, pam_ops
 
 
+FULLY_PAM = False        # softmax and LayerNorm through the package too (the reference's multiplication-free recipe)
+
+
+def _softmax(s):
+    return pam_amd.softmax(s, dim=-1, approx_bwd=True) if FULLY_PAM else torch.softmax(s, -1)
+
+
+def _norm(d):
+    return pam_amd.LayerNorm(d, approx_bwd=True) if FULLY_PAM else torch.nn.LayerNorm(d)
+
+
 class Attention(torch.nn.Module):
     def __init__(self, d, heads):
         super().__init__()
@@ -24,18 +35,18 @@ class Attention(torch.nn.Module):
         s = pam_amd.bmm(q, k.transpose(1, 2), approx_bwd=True)
         if causal:
             s = s.masked_fill(torch.ones(T, S, dtype=torch.bool, device=x.device).triu(1), float("-inf"))
-        o = pam_amd.bmm(torch.softmax(s, -1), v, approx_bwd=True)
+        o = pam_amd.bmm(_softmax(s), v, approx_bwd=True)
         return self.o(o.view(B, H, T, dh).transpose(1, 2).reshape(B, T, D))
 
 
 class Layer(torch.nn.Module):
     def __init__(self, d, ffn, heads, cross):
         super().__init__()
-        self.sa = Attention(d, heads); self.n1 = torch.nn.LayerNorm(d)
+        self.sa = Attention(d, heads); self.n1 = _norm(d)
         self.ca = Attention(d, heads) if cross else None
-        self.n2 = torch.nn.LayerNorm(d) if cross else None
+        self.n2 = _norm(d) if cross else None
         self.f1 = pam_amd.Linear(d, ffn, approx_bwd=True); self.f2 = pam_amd.Linear(ffn, d, approx_bwd=True)
-        self.n3 = torch.nn.LayerNorm(d)
+        self.n3 = _norm(d)
 
     def forward(self, x, mem=None):
         x = self.n1(x + self.sa(x, x, causal=mem is not None))
@@ -114,3 +125,46 @@ def test_full_size_step_runs():
     assert sum(float(g.abs().sum()) for g in grads.values()) > 0
     loss2, grads2 = _step(model, src, tgt, lab)
     assert torch.equal(loss, loss2) and all(torch.equal(grads[n], grads2[n]) for n in grads)
+
+
+@pytest.mark.gpu
+def test_fully_pam_recipe_trains(oracle, monkeypatch):
+    """The multiplication-free recipe end to end: PAM linears and attention products, PAM softmax
+    (single kernel with its gradient) and LayerNorm, the op-table cross entropy and the PAM Adam
+    kernel, wired through the configuration hooks.  A few steps on a small model: the first step
+    agrees with an oracle-backed CPU run, the loss falls, and a rerun gives identical bits."""
+    from pam_amd import factories, optim
+    from test_host_api import OracleKernels
+    import sys
+    mod = sys.modules[__name__]
+    monkeypatch.setattr(mod, "FULLY_PAM", True)
+    ops = factories.get_function_dict("pam")
+    src, tgt, lab = _data(101, 8, 12, 3)
+
+    def run(device, steps):
+        torch.manual_seed(0)
+        model = EncDec(vocab=101, d=64, ffn=128, heads=4, layers=2).to(device)
+        opt = optim.Adam(model.parameters(), lr=2e-3, betas=(0.9, 0.98), eps=1e-8, opt_functional_cfg="pam")
+        losses, first_grads = [], None
+        for _ in range(steps):
+            model.zero_grad(set_to_none=True)
+            logits = model(src.to(device), tgt.to(device))
+            loss = pam_amd.cross_entropy(logits.view(-1, logits.shape[-1]), lab.to(device).view(-1), None, -100, "mean", 0.0,
+                                         op_dict=ops)
+            loss.backward()
+            if first_grads is None:
+                first_grads = {n: p.grad.detach().cpu().clone() for n, p in model.named_parameters()}
+            opt.step()
+            losses.append(loss.item())
+        return losses, first_grads, {n: p.detach().cpu().clone() for n, p in model.named_parameters()}
+
+    losses, grads, params = run("cuda", 8)
+    assert all(np.isfinite(losses)) and losses[-1] < losses[0] - 0.05, losses
+    losses2, _, params2 = run("cuda", 8)
+    assert losses == losses2 and all(torch.equal(params[n], params2[n]) for n in params)
+    monkeypatch.setattr(cuda_bindings, "cuda_kernels", OracleKernels(oracle))
+    monkeypatch.setattr(pam_ops, "_require_kernel", lambda t, use_kernel: None)
+    losses_c, grads_c, _ = run("cpu", 1)
+    assert abs(losses[0] - losses_c[0]) <= 1e-4 * abs(losses_c[0])
+    for n, gc in grads_c.items():
+        assert (grads[n] - gc).abs().max() <= 2e-3 * gc.abs().max() + 1e-7, n
