@@ -145,6 +145,26 @@ int pam_hip_row_mean_fwd(const float *x, float *y, long rows, long n, float offs
 int pam_hip_layer_norm_fwd(const float *x, const float *weight, const float *bias, float *y, long rows, long n,
                            float eps, float offset, void *stream);
 
+/* ---- convolution without the unfolded matrix (pam/pam_ops.py:118-160) ---------------------- */
+/* The reference computes conv2d as unfold -> transpose copy -> PAM linear, a kh*kw-fold copy of
+ * the input.  These entry points run the same products and sums on the matrix kernel with the
+ * image patches read in place: x[batch][c][h][w] and w[co][c][kh][kw] contiguous, dilation 1,
+ * output size (in + 2 pad - k) / stride + 1.  Sums run over k = (c, i, j) in ascending order in
+ * the chunks pam_hip_gemm_plan(batch, co, ho*wo, c*kh*kw) reports. */
+size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
+                                      long stride_h, long stride_w, long pad_h, long pad_w, int weight_gradient, float offset);
+/* y[batch][co][ho][wo] = sum_k x_patch (*) (w (*) offset)           replaces pam.conv2d's forward */
+int pam_hip_conv2d_fwd(const float *x, const float *w, float *y, long batch, long c, long h, long wd, long co, long kh, long kw,
+                       long stride_h, long stride_w, long pad_h, long pad_w, float offset,
+                       void *workspace, size_t workspace_bytes, void *stream);
+/* dw[batch][co][c*kh*kw]: each image's contribution to the weight gradient (the caller sums over
+ * the batch, as autograd does for the reference's broadcast weight).  exact == 0: the
+ * approximate gradient sum_l x_patch (*) (dy (*) offset) (pam/cuda_bindings.py:160-161);
+ * exact != 0: sum_l pam_bwd(w, x_patch, dy) (:162-164), w required. */
+int pam_hip_conv2d_bwd_weight(const float *x, const float *dy, const float *w, float *dw, long batch, long c, long h, long wd,
+                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                              int exact, float offset, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- optimizer step ---------------------------------------------------------------------- */
 /* One Adam update of n parameters in place, every product, the quotient and the square root
  * a PAM op                replaces the op-table arithmetic of the training recipe's optimizer

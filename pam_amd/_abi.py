@@ -43,6 +43,9 @@ _SIGNATURES = {
     "pam_hip_standard_bmm": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_matmul_bwd": (_MAT2 * 4 + [_l, _l, _l, _i, _f, _p, _z, _p], _i),
     "pam_hip_pam_bmm_bwd": (_MAT * 4 + [_l, _l, _l, _l, _i, _f, _p, _z, _p], _i),
+    "pam_hip_conv2d_workspace_bytes": ([_l] * 11 + [_i, _f], _z),
+    "pam_hip_conv2d_fwd": ([_p, _p, _p] + [_l] * 11 + [_f, _p, _z, _p], _i),
+    "pam_hip_conv2d_bwd_weight": ([_p, _p, _p, _p] + [_l] * 11 + [_i, _f, _p, _z, _p], _i),
     "pam_hip_adam_step": ([_p, _p, _p, _p, _z, _f, _f, _f, _f, _f, _f, _i, _f, _f, _p], _i),
     "pam_hip_rowop_workspace_bytes": ([], _z),
     "pam_hip_softmax_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
@@ -350,3 +353,43 @@ def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, d
             _call("pam_hip_adam_step", p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), float(beta1),
                   float(one_minus_beta1), float(beta2), float(one_minus_beta2), float(eps), float(decay or 0.0),
                   int(bool(decay)), float(step_size), float(offset), _stream())
+
+
+def _conv_geometry(X, W, stride, padding):
+    if X.dim() != 4 or W.dim() != 4 or X.shape[1] != W.shape[1]:
+        raise ValueError("conv2d: expected X[batch, c, h, w] and W[co, c, kh, kw]")
+    batch, c, h, w = X.shape
+    co, _, kh, kw = W.shape
+    return [batch, c, h, w, co, kh, kw, stride[0], stride[1], padding[0], padding[1]]
+
+
+def conv2d_fwd(X, W, stride, padding, offset):
+    """Y[batch, co, ho, wo] for contiguous fp32 GPU tensors, dilation 1; the image patches are read in place."""
+    _check(X, W)
+    X, W = X.contiguous(), W.contiguous()
+    geo = _conv_geometry(X, W, stride, padding)
+    batch, c, h, w, co, kh, kw, sh, sw, ph, pw = geo
+    ho, wo = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
+    Y = torch.empty((batch, co, ho, wo), dtype=torch.float32, device=X.device)
+    if Y.numel():
+        with torch.cuda.device(X.device):
+            nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 0, float(offset))
+            ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=X.device)
+            _call("pam_hip_conv2d_fwd", X.data_ptr(), W.data_ptr(), Y.data_ptr(), *geo, float(offset), ws.data_ptr(), nbytes, _stream())
+    return Y
+
+
+def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset):
+    """Per-image weight gradients [batch, co, c*kh*kw]; W is only read by the exact variant."""
+    _check(X, dY, W)
+    X, dY, W = X.contiguous(), dY.contiguous(), W.contiguous()
+    geo = _conv_geometry(X, W, stride, padding)
+    batch, c, _, _, co, kh, kw = geo[:7]
+    dW = torch.empty((batch, co, c * kh * kw), dtype=torch.float32, device=X.device)
+    if dW.numel():
+        with torch.cuda.device(X.device):
+            nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 1, float(offset))
+            ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=X.device)
+            _call("pam_hip_conv2d_bwd_weight", X.data_ptr(), dY.data_ptr(), W.data_ptr(), dW.data_ptr(), *geo,
+                  int(bool(exact)), float(offset), ws.data_ptr(), nbytes, _stream())
+    return dW

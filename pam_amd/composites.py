@@ -7,7 +7,8 @@ reference.  Same names and keyword arguments.
 Reductions over the last dimension of a contiguous GPU tensor take the single-kernel path of
 `pam_amd.fused` (softmax always, the others when no autograd graph is recorded); every other
 call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
-the single-kernel path off.
+the single-kernel path off.  conv2d on GPU tensors runs on the matrix kernel with the image
+patches read in place instead of unfolded (`implicit_conv = False` switches that off).
 """
 import math
 
@@ -21,6 +22,7 @@ __all__ = ["mean", "softmax", "logsumexp", "log_softmax", "layer_norm", "LayerNo
 
 _LOG2_E = math.log2(math.e)
 fused_rows = True
+implicit_conv = True
 
 
 def _fused(x, dim, use_kernel, *grad_sources):
@@ -161,6 +163,9 @@ def conv2d(X, W, bias=None, stride=1, padding=0, dilation=1, *, offset=None, app
     batch = X.shape[0]
     c_out, _, kh, kw = W.shape
     padding, stride, (h_out, w_out) = _conv_geometry(X.shape[2:], (kh, kw), stride, padding)
+    if implicit_conv and use_kernel and fused.conv_in_place(X, W, dilation, approx_bwd):
+        out = fused.conv2d(X, W, stride, padding, offset, approx_bwd)        # patches read in place
+        return out if bias is None else out + bias.view((1, -1, 1, 1))
     patches = torch.nn.functional.unfold(X, (kh, kw), padding=padding, stride=stride, dilation=dilation)
     _, patch_len, locations = patches.shape                    # [N, C kh kw, L]
     rows = patches.transpose(1, 2).contiguous().view(-1, patch_len)

@@ -46,14 +46,24 @@ using namespace pamdev;
 namespace {
 
 enum { MODE_PAM = 0, MODE_STD = 1, MODE_BWD_DL = 2, MODE_BWD_DR = 3 };
-enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2 };   // k contiguous / row contiguous / any strides
+enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3 };   // k contiguous / row contiguous / any strides / image patches
 
 constexpr int KGRAN = 32;         // k ranges handed to work-groups are multiples of this
 constexpr int PAD = 4;
 
 struct Operand { const float* p; long sb, sr, sk; };    // batch, row (the non-k index), k strides
+
+// The right operand as the patches of an image, never materialised (the reference unfolds them
+// into a [C kh kw, Ho Wo] matrix per image, pam/pam_ops.py:118-160): entry (k, l) of that matrix
+// is x[c, h0(l) + di(k), w0(l) + dj(k)], zero outside the image.  Two small tables hold, per k
+// and per l, the address part and the coordinates: {c H W + di W + dj, di << 16 | dj} and
+// {h0 W + w0, h0 << 16 | (w0 & 0xffff)}.  `transposed` exchanges the roles of the operand's two
+// indices (the matrix is then [Ho Wo, C kh kw]: the weight-gradient product).
+struct ConvGeom { const int2* ktab; const int2* ltab; int H, W; int transposed; };
+
 struct GemmArgs {
     Operand L, R;
+    ConvGeom cv;
     const float* D; long d_sb, d_sr, d_sc;
     float* Y; long y_sb, y_sr, y_sc;
     int M, N, K;
@@ -105,12 +115,37 @@ template <int ROWS, int NT, int KIND, int BK>
 struct TileLoader {
     static constexpr int kVecs = ROWS * BK / 4 / NT;      // float4 per lane (vector kinds)
     static constexpr int kElems = ROWS * BK / NT;         // scalars per lane (generic kind)
-    static_assert(ROWS * BK % (4 * NT) == 0, "tile must divide over the work-group");
+    static_assert(ROWS * BK % (4 * NT) == 0 && NT % ROWS == 0, "tile must divide over the work-group");
     float4 v[kVecs > 0 ? kVecs : 1];
+    int2 fixed; bool have_fixed = false;          // LOAD_CONV: the lane's own table entry
 
-    __device__ __forceinline__ void load(const Operand& op, const float* base, int row0, int nrows, int k0, int kend, int tid)
+    __device__ __forceinline__ void load(const Operand& op, const float* base, int row0, int nrows, int k0, int kend, int tid,
+                                         const ConvGeom& cv)
     {
-        if (KIND == LOAD_KVEC) {
+        if (KIND == LOAD_CONV) {
+            float* s = reinterpret_cast<float*>(v);
+            // Every element of a lane has the same row (NT is a multiple of ROWS): one table entry,
+            // fetched once per work-group.  The k index is the same for a whole wavefront (ROWS is
+            // the wavefront size), so its table entry comes through the scalar unit.
+            if (!have_fixed) {
+                const int row = min(row0 + tid % ROWS, nrows - 1);
+                fixed = cv.transposed ? cv.ktab[row] : cv.ltab[row];
+                have_fixed = true;
+            }
+            const int kwave = __builtin_amdgcn_readfirstlane(tid / ROWS);
+            // the tables are written before the launch and only read here: constant address space
+            typedef const __attribute__((address_space(4))) int* ConstTable;
+            ConstTable mtab = (ConstTable)(cv.transposed ? cv.ltab : cv.ktab);
+#pragma unroll
+            for (int i = 0; i < kElems; ++i) {
+                const int kk = min(k0 + kwave + i * (NT / ROWS), kend - 1);
+                const int2 moving = make_int2(mtab[2 * kk], mtab[2 * kk + 1]);
+                const int2 ke = cv.transposed ? fixed : moving, le = cv.transposed ? moving : fixed;
+                const int h = (le.y >> 16) + (ke.y >> 16), w = (int)(short)(le.y & 0xffff) + (ke.y & 0xffff);
+                const bool inside = (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
+                s[i] = inside ? base[ke.x + le.x] : 0.0f;
+            }
+        } else if (KIND == LOAD_KVEC) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
@@ -172,7 +207,7 @@ struct TileLoader {
                 w.x = st.one(v[i].x); w.y = st.one(v[i].y); w.z = st.one(v[i].z); w.w = st.one(v[i].w);
                 *reinterpret_cast<uint4*>(lds + (id / (ROWS / 4)) * LD + (id % (ROWS / 4)) * 4) = w;
             }
-        } else {
+        } else {                                    // LOAD_ANY and LOAD_CONV: lane-consecutive rows
             const float* s = reinterpret_cast<const float*>(v);
 #pragma unroll
             for (int i = 0; i < kElems; ++i) {
@@ -274,8 +309,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
     };
 
     if (ktiles > 0) {
-        ll.load(g.L, lbase, row0, g.M, kbegin, kend, tid);
-        rl.load(g.R, rbase, col0, g.N, kbegin, kend, tid);
+        ll.load(g.L, lbase, row0, g.M, kbegin, kend, tid, g.cv);
+        rl.load(g.R, rbase, col0, g.N, kbegin, kend, tid, g.cv);
         stage(0);
     }
     __syncthreads();
@@ -284,8 +319,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
         const int cur = t & 1;
         const int k0 = kbegin + t * BK;
         if (t + 1 < ktiles) {
-            ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid);
-            rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid);
+            ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid, g.cv);
+            rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid, g.cv);
         }
         const int kcount = min(BK, kend - k0);
         uint32_t verdict = 0;                     // 0 plain loop, 1 zeros present, 2 guarded
@@ -492,6 +527,9 @@ void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, 
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
+    if constexpr (MODE == MODE_PAM || MODE == MODE_BWD_DL) {           // image patches as the right operand
+        PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_RVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_ANY, LOAD_CONV)
+    }
 #undef PAM_GEMM_CASE
 }
 
@@ -506,7 +544,7 @@ void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& 
 int gemm(const char* what, int mode, long batch, long M, long N, long K,
          const float* l, long l_sb, long l_sr, long l_sc, const float* r, long r_sb, long r_sr, long r_sc,
          const float* d, long d_sb, long d_sr, long d_sc, float* y, long y_sb, long y_sr, long y_sc,
-         float offset, void* workspace, size_t workspace_bytes, void* stream)
+         float offset, void* workspace, size_t workspace_bytes, void* stream, const ConvGeom* conv = nullptr)
 {
     if (batch < 0 || M < 0 || N < 0 || K < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: negative size", what);
     if (batch == 0 || M == 0 || N == 0) return PAM_HIP_OK;
@@ -530,8 +568,10 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     g.ksplit = p.ksplit; g.kchunk = p.kchunk;
     g.off = offset; g.has_off = (mode != MODE_STD && offset != 1.0f) ? 1 : 0;
 
+    g.cv = conv ? *conv : ConvGeom{nullptr, nullptr, 0, 0, 0};
+
     int lk = load_kind(l_sr, l_sc, l_sb, l, M, K);
-    int rk = load_kind(r_sc, r_sr, r_sb, r, N, K);
+    int rk = conv ? LOAD_CONV : load_kind(r_sc, r_sr, r_sb, r, N, K);
     float* partial = (float*)workspace;
     switch (mode) {
     case MODE_PAM: launch_mode<MODE_PAM>(p, lk, rk, st, g, batch, partial); break;
@@ -545,6 +585,69 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
                            partial, p.ksplit, slab, y, y_sb, y_sr, y_sc, (int)M, (int)N);
     }
     return pamhost::check_launch(what);
+}
+
+// ---------------------------------------------------------------- convolution as a product with image patches
+struct ConvShape { long batch, c, h, w, co, kh, kw, sh, sw, ph, pw, ho, wo; long K() const { return c * kh * kw; } long L() const { return ho * wo; } };
+
+__global__ __launch_bounds__(256) void conv_tables_kernel(int2* __restrict__ ktab, int2* __restrict__ ltab, int K, int L,
+                                                         int kh, int kw, int H, int W, int wo, int sh, int sw, int ph, int pw)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx < K) {
+        const int c = idx / (kh * kw), rem = idx % (kh * kw), i = rem / kw, j = rem % kw;
+        ktab[idx] = make_int2(c * H * W + i * W + j, (i << 16) | j);
+    }
+    if (idx < L) {
+        const int h0 = (idx / wo) * sh - ph, w0 = (idx % wo) * sw - pw;
+        ltab[idx] = make_int2(h0 * W + w0, (int)(((unsigned)h0 << 16) | ((unsigned)w0 & 0xffffu)));
+    }
+}
+
+__global__ __launch_bounds__(256) void scale_kernel(const float* __restrict__ in, float* __restrict__ out, size_t n, float off)
+{
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) out[i] = pam_mul(in[i], off);
+}
+
+size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+int conv_shape(const char* what, ConvShape& s)
+{
+    if (s.batch < 0 || s.c <= 0 || s.h <= 0 || s.w <= 0 || s.co <= 0 || s.kh <= 0 || s.kw <= 0 || s.sh <= 0 || s.sw <= 0 || s.ph < 0 || s.pw < 0)
+        return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: bad geometry", what);
+    s.ho = (s.h + 2 * s.ph - s.kh) / s.sh + 1;             // (in + 2 pad - (k - 1) - 1) / stride + 1 (pam/pam_ops.py:137-138)
+    s.wo = (s.w + 2 * s.pw - s.kw) / s.sw + 1;
+    if (s.h + 2 * s.ph < s.kh || s.w + 2 * s.pw < s.kw) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: kernel larger than the padded image", what);
+    if (s.c * s.h * s.w >= (1L << 31) || s.h >= 32768 || s.w >= 32768 || s.kh >= 32768 || s.kw >= 32768 || s.ph >= 16384 || s.pw >= 16384)
+        return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: image too large for the patch tables", what);
+    return PAM_HIP_OK;
+}
+
+// workspace: [k table][l table][operand scaled by the offset, if any][split-k partial tiles]
+struct ConvSpace { size_t tables, scaled, total; };
+ConvSpace conv_space(const ConvShape& s, bool weight_gradient, bool has_off)
+{
+    ConvSpace w;
+    w.tables = align256((size_t)(s.K() + s.L()) * sizeof(int2));
+    size_t scaled_elems = !has_off ? 0 : weight_gradient ? (size_t)s.batch * s.co * s.L() : (size_t)s.co * s.K();
+    w.scaled = align256(scaled_elems * sizeof(float));
+    size_t split = weight_gradient ? pam_hip_gemm_workspace_bytes(s.batch, s.co, s.K(), s.L())
+                                   : pam_hip_gemm_workspace_bytes(s.batch, s.co, s.L(), s.K());
+    w.total = w.tables + w.scaled + split;
+    return w;
+}
+
+int conv_prepare(const char* what, const ConvShape& s, const ConvSpace& sp, void* workspace, size_t workspace_bytes,
+                 hipStream_t st, ConvGeom& cv, bool transposed)
+{
+    if (!workspace || workspace_bytes < sp.total)
+        return pamhost::fail(PAM_HIP_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", what, sp.total);
+    int2* ktab = (int2*)workspace; int2* ltab = ktab + s.K();
+    const long n = s.K() > s.L() ? s.K() : s.L();
+    hipLaunchKernelGGL(conv_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, ktab, ltab, (int)s.K(), (int)s.L(),
+                       (int)s.kh, (int)s.kw, (int)s.h, (int)s.w, (int)s.wo, (int)s.sh, (int)s.sw, (int)s.ph, (int)s.pw);
+    cv = ConvGeom{ktab, ltab, (int)s.h, (int)s.w, transposed ? 1 : 0};
+    return PAM_HIP_OK;
 }
 
 }  // namespace
@@ -616,6 +719,77 @@ int pam_hip_pam_bmm_bwd(PAM_HIP_MAT(l), PAM_HIP_MAT(r), PAM_HIP_MAT(mo), PAM_HIP
 {
     return gemm("pam_bmm_bwd", delta_l ? MODE_BWD_DL : MODE_BWD_DR, batch, m, n, k, l, l_sb, l_sr, l_sc, r, r_sb, r_sr, r_sc,
                 mo, mo_sb, mo_sr, mo_sc, dm, dm_sb, dm_sr, dm_sc, offset, workspace, workspace_bytes, stream);
+}
+
+size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
+                                      long stride_h, long stride_w, long pad_h, long pad_w, int weight_gradient, float offset)
+{
+    ConvShape s{batch, c, h, w, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    if (conv_shape("conv2d_workspace_bytes", s) != PAM_HIP_OK || batch == 0) return 0;
+    return conv_space(s, weight_gradient != 0, offset != 1.0f).total;
+}
+
+int pam_hip_conv2d_fwd(const float* x, const float* w, float* y, long batch, long c, long h, long wd, long co, long kh, long kw,
+                       long stride_h, long stride_w, long pad_h, long pad_w, float offset,
+                       void* workspace, size_t workspace_bytes, void* stream)
+{
+    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    int rc = conv_shape("conv2d_fwd", s);
+    if (rc != PAM_HIP_OK) return rc;
+    if (batch == 0) return PAM_HIP_OK;
+    if (!x || !w || !y) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_fwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const bool has_off = offset != 1.0f;
+    ConvSpace sp = conv_space(s, false, has_off);
+    ConvGeom cv;
+    rc = conv_prepare("conv2d_fwd", s, sp, workspace, workspace_bytes, st, cv, false);
+    if (rc != PAM_HIP_OK) return rc;
+    // the reference folds the offset into the weights (the right operand of its product); here the
+    // weights are the left operand, so they are scaled once up front
+    const float* wl = w;
+    if (has_off) {
+        float* scaled = (float*)((char*)workspace + sp.tables);
+        size_t n = (size_t)co * s.K();
+        hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, w, scaled, n, offset);
+        wl = scaled;
+    }
+    const long K = s.K(), L = s.L();
+    // per image: Y[co, l] = sum_k W[co, k] (*) patches[k, l]
+    return gemm("conv2d_fwd", MODE_PAM, batch, co, L, K, wl, 0, K, 1, x, c * h * wd, 0, 0, nullptr, 0, 0, 0,
+                y, co * L, L, 1, 1.0f, (char*)workspace + sp.tables + sp.scaled, workspace_bytes - sp.tables - sp.scaled, stream, &cv);
+}
+
+int pam_hip_conv2d_bwd_weight(const float* x, const float* dy, const float* w, float* dw, long batch, long c, long h, long wd,
+                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                              int exact, float offset, void* workspace, size_t workspace_bytes, void* stream)
+{
+    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    int rc = conv_shape("conv2d_bwd_weight", s);
+    if (rc != PAM_HIP_OK) return rc;
+    if (batch == 0) return PAM_HIP_OK;
+    if (!x || !dy || !dw || (exact && !w)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_bwd_weight: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const bool scale = offset != 1.0f && !exact;
+    ConvSpace sp = conv_space(s, true, scale);
+    ConvGeom cv;
+    rc = conv_prepare("conv2d_bwd_weight", s, sp, workspace, workspace_bytes, st, cv, true);
+    if (rc != PAM_HIP_OK) return rc;
+    const long K = s.K(), L = s.L();
+    void* rest = (char*)workspace + sp.tables + sp.scaled; size_t rest_bytes = workspace_bytes - sp.tables - sp.scaled;
+    if (exact)        // dW[co, k] = sum_l pam_bwd(W[co, k], patches[k, l], dY[co, l]); the offset goes with the patches
+        return gemm("conv2d_bwd_weight", MODE_BWD_DL, batch, co, K, L, dy, co * L, L, 1, x, c * h * wd, 0, 0, w, 0, K, 1,
+                    dw, co * K, K, 1, offset, rest, rest_bytes, stream, &cv);
+    // approximate: dW[co, k] = sum_l patches[k, l] (*) (dY[co, l] (*) offset), the gradient scaled once up front
+    const float* dl = dy;
+    if (scale) {
+        float* scaled = (float*)((char*)workspace + sp.tables);
+        size_t n = (size_t)batch * co * L;
+        size_t blocks = (n + 1023) / 1024; if (blocks > (1u << 20)) blocks = 1u << 20;
+        hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, dy, scaled, n, offset);
+        dl = scaled;
+    }
+    return gemm("conv2d_bwd_weight", MODE_PAM, batch, co, K, L, dl, co * L, L, 1, x, c * h * wd, 0, 0, nullptr, 0, 0, 0,
+                dw, co * K, K, 1, 1.0f, rest, rest_bytes, stream, &cv);
 }
 
 }  // extern "C"

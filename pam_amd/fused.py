@@ -12,6 +12,8 @@ contiguous, reduced dimension last, not empty.
 """
 import torch
 
+from . import _abi
+from . import cuda_bindings
 from ._abi import HipRowKernels
 from .cuda_bindings import _both, _offset_value
 
@@ -90,3 +92,59 @@ def layer_norm(x, n, weight, bias, eps, offset=None):
     w = None if weight is None else weight.detach().contiguous().view(-1)
     b = None if bias is None else bias.detach().contiguous().view(-1)
     return row_kernels.layer_norm_fwd(x.reshape(-1, n), w, b, eps, _offset_value(offset)).view(x.shape)
+
+
+# ---------------------------------------------------------------- convolution on image patches read in place
+
+def conv_in_place(X, W, dilation, approx_bwd):
+    """True when conv2d can run on the matrix kernel without unfolding X: fp32 GPU tensors,
+    dilation 1, and no exact gradient with respect to X wanted (that one needs the patches as
+    a stored operand)."""
+    if not (isinstance(X, torch.Tensor) and isinstance(W, torch.Tensor) and X.is_cuda and W.is_cuda):
+        return False
+    if X.dtype != torch.float32 or W.dtype != torch.float32 or X.dim() != 4 or W.dim() != 4 or X.numel() == 0:
+        return False
+    if dilation not in (1, (1, 1), [1, 1]):
+        return False
+    approx_x, _ = _both(approx_bwd)
+    return approx_x or not (torch.is_grad_enabled() and X.requires_grad)
+
+
+class conv2d_autograd(torch.autograd.Function):
+    """conv2d as W (x) patches(X) per image.  The reference's product is patches (x) W^T
+    (pam/pam_ops.py:118-160); PAM products commute, and the offset, which the reference folds
+    into the weights, is applied to them before the product, so every term is the same."""
+
+    @staticmethod
+    def forward(ctx, X, W, stride, padding, offset, approx_bwd):
+        ctx.stride, ctx.padding = stride, padding
+        ctx.offset = _offset_value(offset)
+        ctx.approx_bwd = approx_bwd
+        ctx.save_for_backward(X, W)
+        return _abi.conv2d_fwd(X, W, stride, padding, ctx.offset)
+
+    @staticmethod
+    def backward(ctx, dY):
+        X, W = ctx.saved_tensors
+        approx_x, approx_w = _both(ctx.approx_bwd)       # the reference's A is the patch matrix, its B the weights
+        k, off = cuda_bindings.cuda_kernels, ctx.offset
+        dY = dY.contiguous()
+        dX = dW = None
+        if ctx.needs_input_grad[1]:
+            per_image = _abi.conv2d_bwd_weight(X, dY, W, ctx.stride, ctx.padding, not approx_w, off)
+            dW = per_image.sum(0).view(W.shape)
+        if ctx.needs_input_grad[0]:
+            if not approx_x:
+                raise RuntimeError("exact gradient with respect to the convolution input needs the unfolded path")
+            batch, co = dY.shape[:2]
+            W2 = W.reshape(co, -1)
+            if off != 1.0:
+                W2 = k.pam_fwd(W2, torch.tensor(off, dtype=torch.float32, device=W.device).expand_as(W2), 1.0)
+            # gradient of the patch matrix, then the overlap-add that is unfold's gradient
+            d_patches = k.pam_bmm_fwd(W2.t().unsqueeze(0).expand(batch, -1, -1), dY.view(batch, co, -1), False, True, 1.0)
+            dX = torch.nn.functional.fold(d_patches, X.shape[2:], W.shape[2:], padding=ctx.padding, stride=ctx.stride)
+        return dX, dW, None, None, None, None
+
+
+def conv2d(X, W, stride, padding, offset=None, approx_bwd=False):
+    return conv2d_autograd.apply(X, W, tuple(stride), tuple(padding), offset, approx_bwd)

@@ -1,0 +1,129 @@
+"""conv2d on the matrix kernel with the image patches read in place: against the oracle's
+product on the unfolded matrix (bit for bit, same accumulation plan), against the unfolded
+composition on the same GPU (same terms, other summation grouping), and its gradients."""
+import numpy as np
+import pytest
+import torch
+
+import pam_amd
+from pam_amd import _abi, composites
+from _util import assert_same_bits
+
+pytestmark = pytest.mark.gpu
+OFF = 1.0552
+
+CASES = [
+    # batch, c, h, w, co, kh, kw, stride, padding
+    (2, 3, 9, 8, 5, 3, 3, (1, 1), (1, 1)),
+    (3, 6, 12, 10, 70, 3, 5, (2, 1), (0, 2)),
+    (2, 4, 16, 16, 8, 4, 4, (4, 4), (0, 0)),          # non-overlapping patches (patch embedding)
+    (1, 20, 7, 7, 33, 1, 1, (1, 1), (0, 0)),
+    (2, 16, 32, 32, 64, 3, 3, (1, 1), (1, 1)),
+]
+
+
+def _inputs(case, seed, specials=False):
+    batch, c, h, w, co, kh, kw, stride, padding = case
+    rng = np.random.RandomState(seed)
+    X = rng.standard_normal((batch, c, h, w)).astype(np.float32)
+    W = (rng.standard_normal((co, c, kh, kw)) * 0.1).astype(np.float32)
+    if specials:
+        flat = X.reshape(-1)
+        flat[rng.choice(flat.size, 6, replace=False)] = [0.0, -0.0, 1e-40, -3e38, np.inf, np.nan]
+    return X, W
+
+
+def _unfold(X, case):
+    _, _, _, _, _, kh, kw, stride, padding = case
+    return torch.nn.functional.unfold(torch.from_numpy(X), (kh, kw), padding=padding, stride=stride).numpy()   # [B, K, L]
+
+
+def _plan(batch, m, n, k):
+    return _abi.gemm_plan(batch, m, n, k)[0]
+
+
+@pytest.mark.parametrize("off", [None, OFF])
+@pytest.mark.parametrize("case", CASES)
+def test_forward_against_oracle(oracle, case, off):
+    batch, c, h, w, co, kh, kw, stride, padding = case
+    for specials in (False, True):
+        X, W = _inputs(case, 1, specials)
+        P = _unfold(X, case)
+        K, L = P.shape[1:]
+        W2 = W.reshape(co, K)
+        Wl = W2 if off is None else oracle.pam(W2, np.float32(off))         # the offset goes with the weights
+        want = oracle.gemm(np.broadcast_to(Wl, (batch, co, K)), P, kchunk=_plan(batch, co, L, K))
+        got = _abi.conv2d_fwd(torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda(), stride, padding, 1.0 if off is None else off)
+        assert got.shape[2] * got.shape[3] == L
+        assert_same_bits(got.cpu().numpy().reshape(batch, co, L), want, f"conv forward {case} specials={specials}")
+
+
+@pytest.mark.parametrize("off", [None, OFF])
+@pytest.mark.parametrize("case", CASES[:4])
+def test_weight_gradient_against_oracle(oracle, case, off):
+    batch, c, h, w, co, kh, kw, stride, padding = case
+    X, W = _inputs(case, 2)
+    P = _unfold(X, case)
+    K, L = P.shape[1:]
+    dY = (np.random.RandomState(3).standard_normal((batch, co, L)) * 1e-2).astype(np.float32)
+    Xd, Wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
+    dYd = torch.from_numpy(dY).cuda().view(batch, co, *_abi.conv2d_fwd(Xd, Wd, stride, padding, 1.0).shape[2:])
+    Pt = np.ascontiguousarray(P.transpose(0, 2, 1))                          # [B, L, K]
+    plan = _plan(batch, co, K, L)
+    dl = dY if off is None else oracle.pam(dY, np.float32(off))
+    want = oracle.gemm(dl, Pt, kchunk=plan)
+    got = _abi.conv2d_bwd_weight(Xd, dYd, Wd, stride, padding, False, 1.0 if off is None else off)
+    assert_same_bits(got.cpu().numpy(), want, f"approximate weight gradient {case}")
+    want = oracle.gemm(dY, Pt, mode=oracle.MODE_BWD_DELTA_L, D=np.broadcast_to(W.reshape(co, K), (batch, co, K)), offset=off, kchunk=plan)
+    got = _abi.conv2d_bwd_weight(Xd, dYd, Wd, stride, padding, True, 1.0 if off is None else off)
+    assert_same_bits(got.cpu().numpy(), want, f"exact weight gradient {case}")
+
+
+def _close(a, b, tol=3e-6):
+    return (a - b).abs().max().item() <= tol * b.abs().max().item()
+
+
+@pytest.mark.parametrize("approx", [True, (True, False)])
+def test_module_path_matches_unfolded_composition(approx):
+    """pam.conv2d / pam.Conv2d with patches read in place against the unfold + linear chain on the
+    same GPU: values and both gradients agree up to the grouping of the sums."""
+    torch.manual_seed(0)
+    X = torch.randn(4, 6, 14, 11, device="cuda"); W = torch.randn(10, 6, 3, 3, device="cuda") * 0.2; b = torch.randn(10, device="cuda")
+    g = torch.randn(4, 10, 7, 11, device="cuda")
+    res = {}
+    for implicit in (True, False):
+        composites.implicit_conv = implicit
+        try:
+            Xr, Wr = X.clone().requires_grad_(), W.clone().requires_grad_()
+            Y = pam_amd.conv2d(Xr, Wr, b, stride=(2, 1), padding=1, offset=OFF, approx_bwd=approx)
+            Y.backward(g)
+            res[implicit] = (Y.detach(), Xr.grad, Wr.grad)
+        finally:
+            composites.implicit_conv = True
+    assert res[True][0].is_contiguous()
+    for a, c in zip(res[True], res[False]):
+        assert a.shape == c.shape and _close(a, c)
+    # an exact gradient with respect to the input keeps the unfolded path
+    Xr = X.clone().requires_grad_()
+    pam_amd.conv2d(Xr, W, None, padding=1, approx_bwd=False).sum().backward()
+    assert Xr.grad is not None and torch.isfinite(Xr.grad).all()
+    # no gradient wanted for the input (first layer): in place whatever the flags
+    Wr = W.clone().requires_grad_()
+    pam_amd.conv2d(X, Wr, None, padding=1, approx_bwd=False).sum().backward()
+    assert Wr.grad is not None and torch.isfinite(Wr.grad).all()
+
+
+def test_conv_module_against_torch_on_exact_products():
+    """Power-of-two weights make every PAM product exact (pam/test_pam.py:151-170): the layer equals F.conv2d."""
+    torch.manual_seed(1)
+    X1 = (torch.randint(-1024, 1024, (5, 13, 15, 17), device="cuda") / 64.0).requires_grad_()
+    conv = pam_amd.Conv2d(13, 19, (3, 5), padding=(1, 2), stride=(1, 2), approx_bwd=True).cuda()
+    with torch.no_grad():
+        conv.weight.copy_(2.0 ** torch.randint(-8, 8, conv.weight.shape, device="cuda").float())
+    X2 = X1.detach().clone().requires_grad_()
+    Y1 = conv(X1); Y1.sum().backward()
+    Y2 = torch.nn.functional.conv2d(X2, conv.weight.detach(), conv.bias.detach(), padding=(1, 2), stride=(1, 2)); Y2.sum().backward()
+    assert _close(Y1, Y2, 2e-6) and _close(X1.grad, X2.grad, 2e-6)
+    Wt = conv.weight.detach().clone().requires_grad_()
+    torch.nn.functional.conv2d(X2.detach(), Wt, None, padding=(1, 2), stride=(1, 2)).sum().backward()
+    assert _close(conv.weight.grad, Wt.grad, 2e-6)
