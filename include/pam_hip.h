@@ -135,8 +135,9 @@ int pam_hip_softmax_fwd(const float *x, float *y, float *row_sum, float *shift, 
 int pam_hip_softmax_bwd(const float *x, const float *dy, const float *row_sum, const float *shift, float *dx,
                         long rows, long n, float offset, int approx_a, int approx_b, int approx_exp, void *stream);
 /* lse[rows] = logsumexp(x) over the last dim and/or log_softmax[rows][n] = x - lse (either
- * pointer may be NULL)                    replaces pam.logsumexp / pam.log_softmax (:331-347) */
-int pam_hip_logsumexp_fwd(const float *x, float *lse, float *log_softmax, long rows, long n, float offset,
+ * pointer may be NULL); the global shift goes to shift[0] if not NULL
+ *                                          replaces pam.logsumexp / pam.log_softmax (:331-347) */
+int pam_hip_logsumexp_fwd(const float *x, float *lse, float *log_softmax, float *shift, long rows, long n, float offset,
                           void *workspace, size_t workspace_bytes, void *stream);
 /* y[rows] = sum(x[row]) (/) n             replaces pam.mean over the last dim (:288-302) */
 int pam_hip_row_mean_fwd(const float *x, float *y, long rows, long n, float offset, void *stream);
@@ -144,6 +145,16 @@ int pam_hip_row_mean_fwd(const float *x, float *y, long rows, long n, float offs
  *                                          replaces pam.layer_norm (:350-378) */
 int pam_hip_layer_norm_fwd(const float *x, const float *weight, const float *bias, float *y, long rows, long n,
                            float eps, float offset, void *stream);
+/* Gradients of the two above for rows of at most 1024 values, the chain autograd runs over the
+ * unfused ops (pam/cuda_bindings.py:43-57, 78-97, 224-239, 262-276) in one kernel each.
+ * logsumexp_bwd: grad is [rows] (log_softmax == 0) or [rows][n] (the gradient of x - logsumexp(x));
+ * shift is the forward's global shift.  layer_norm_bwd: dw_terms[rows][n], if not NULL, receives
+ * the per-element terms whose sum over rows is the weight gradient (the bias gradient is the sum
+ * of dy over rows). */
+int pam_hip_logsumexp_bwd(const float *x, const float *grad, const float *shift, float *dx, long rows, long n,
+                          int log_softmax, float offset, int approx_a, int approx_b, int approx_exp, void *stream);
+int pam_hip_layer_norm_bwd(const float *x, const float *weight, const float *dy, float *dx, float *dw_terms, long rows, long n,
+                           float eps, float offset, int approx_a, int approx_b, int approx_exp, void *stream);
 
 /* ---- convolution without the unfolded matrix (pam/pam_ops.py:118-160) ---------------------- */
 /* The reference computes conv2d as unfold -> transpose copy -> PAM linear, a kh*kw-fold copy of

@@ -551,6 +551,94 @@ void pamo_layer_norm_fwd(const float *x, const float *weight, const float *bias,
     }
 }
 
+/* ---- gradients of logsumexp / log_softmax and layer_norm: autograd's chain over the unfused ops
+ * (formulas pam/cuda_bindings.py:43-57, 78-97, 224-239, 262-276; ops pam/pam_ops.py:331-378) ---- */
+typedef struct { float off; int a, b, e; } grad_cfg;
+static float g_mul_da(grad_cfg k, float a, float b, float g) { return k.a ? pam_off(g, b, k.off) : pam_bwd1(a, b, g, k.off); }
+static float g_mul_db(grad_cfg k, float a, float b, float g) { return k.b ? pam_off(g, a, k.off) : pam_bwd1(b, a, g, k.off); }
+static float g_div_da(grad_cfg k, float a, float b, float g)
+{ float inv = pad_off(1.0f, b, k.off); return k.a ? pam_off(inv, g, k.off) : pam_bwd1(a, inv, g, 1.0f); }
+static float g_div_db(grad_cfg k, float a, float b, float g)
+{
+    if (!k.b) return pad_bwd1(a, b, g, k.off);
+    volatile float t = pam_off(pad_off(pad_off(a, b, k.off), b, k.off), g, k.off);
+    return -t;
+}
+static float g_exp2_dx(grad_cfg k, float x, float g)
+{ return k.e ? pam_off(pam_off(exp2_op(x, k.off), LN_2, k.off), g, k.off) : paexp_bwd(x, g, 1.0f, k.off); }
+static float g_log2_dx(grad_cfg k, float x, float g)
+{ return k.e ? pad_off(pad_off(g, x, k.off), LN_2, k.off) : palog_bwd(x, g, 1.0f, k.off); }
+
+/* grad: [rows] for logsumexp, [rows][n] for log_softmax (y = x - logsumexp(x)) */
+void pamo_logsumexp_bwd(const float *x, const float *grad, float shift, float *dx, long rows, long n, int log_softmax,
+                        float off, int approx_a, int approx_b, int approx_exp)
+{
+    grad_cfg k = {off, approx_a, approx_b, approx_exp};
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) {
+        const float *xr = x + r * n;
+        float *e = row_buffer(n);
+        for (long i = 0; i < n; ++i) { volatile float t = scaled_x(xr[i], off, 0) - shift; e[i] = exp2_op(t, off); }
+        float total = row_sum_fixed(e, n);
+        float g_out;
+        if (log_softmax) { volatile float s = row_sum_fixed(grad + r * n, n); g_out = -s; } else g_out = grad[r];
+        volatile float u = shift + log2_op(total, off);
+        float du = g_div_da(k, u, LOG2_E, g_out);
+        float dtotal = g_log2_dx(k, total, du);
+        for (long i = 0; i < n; ++i) {
+            volatile float t = scaled_x(xr[i], off, 0) - shift;
+            float d = g_mul_da(k, xr[i], LOG2_E, g_exp2_dx(k, t, dtotal));
+            if (log_softmax) { volatile float s = grad[r * n + i] + d; d = s; }
+            dx[r * n + i] = d;
+        }
+        free(e);
+    }
+}
+
+/* dx and, if dw_terms is given, the per-element terms whose sum over rows is the weight gradient */
+void pamo_layer_norm_bwd(const float *x, const float *weight, const float *gy, float *dx, float *dw_terms, long rows, long n,
+                         float eps, float off, int approx_a, int approx_b, int approx_exp)
+{
+    grad_cfg k = {off, approx_a, approx_b, approx_exp};
+    #pragma omp parallel for schedule(static)
+    for (long r = 0; r < rows; ++r) {
+        const float *xr = x + r * n, *gr = gy + r * n;
+        float *c = row_buffer(n), *q = row_buffer(n), *g = row_buffer(n), *t = row_buffer(n);
+        float count = (float)n;
+        float s1 = row_sum_fixed(xr, n), mu = pad_off(s1, count, off);
+        for (long i = 0; i < n; ++i) { volatile float d = xr[i] - mu; c[i] = d; q[i] = pam_off(d, d, off); }
+        float s2 = row_sum_fixed(q, n);
+        volatile float v = pad_off(s2, count, off) + eps;
+        float lg = log2_op(v, off), half = pam_off(lg, 0.5f, off);
+        float denom = v == 0.0f ? 0.0f : exp2_op(half, off);
+        for (long i = 0; i < n; ++i) {
+            g[i] = gr[i];
+            if (weight) {
+                float xn = pad_off(c[i], denom, off);
+                if (dw_terms) dw_terms[r * n + i] = g_mul_db(k, xn, weight[i], gr[i]);
+                g[i] = g_mul_da(k, xn, weight[i], gr[i]);
+            }
+            t[i] = g_div_db(k, c[i], denom, g[i]);
+        }
+        float d = row_sum_fixed(t, n);
+        if (v == 0.0f) d = 0.0f;
+        d = g_exp2_dx(k, half, d);
+        d = g_mul_da(k, lg, 0.5f, d);
+        d = g_log2_dx(k, v, d);
+        float ds2 = g_div_da(k, s2, count, d);
+        for (long i = 0; i < n; ++i) {
+            volatile float dc = g_div_da(k, c[i], denom, g[i]);
+            dc = dc + g_mul_da(k, c[i], c[i], ds2);
+            dc = dc + g_mul_db(k, c[i], c[i], ds2);
+            t[i] = dc;
+        }
+        volatile float sdc = row_sum_fixed(t, n);
+        float ds1 = g_div_da(k, s1, count, -sdc);
+        for (long i = 0; i < n; ++i) { volatile float o = t[i] + ds1; dx[r * n + i] = o; }
+        free(c); free(q); free(g); free(t);
+    }
+}
+
 /* One Adam update with PAM ops (submodules/fairseq/fairseq/optim/adam.py:226-252 of the
  * reference tree), the chain of primitive calls written out; in place. */
 void pamo_adam_step(float *p, const float *g, float *m, float *v, size_t n, float beta1, float one_minus_beta1,

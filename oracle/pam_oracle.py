@@ -63,6 +63,9 @@ def lib():
         L.pamo_logsumexp_fwd.argtypes = [_fp, _fp, _fp, cl, cl, cf]
         L.pamo_row_mean_fwd.argtypes = [_fp, _fp, cl, cl, cf]
         L.pamo_layer_norm_fwd.argtypes = [_fp, _fp, _fp, _fp, cl, cl, cf, cf]
+        L.pamo_logsumexp_bwd.argtypes = [_fp, _fp, cf, _fp, cl, cl, ci, cf, ci, ci, ci]
+        L.pamo_layer_norm_bwd.argtypes = [_fp, _fp, _fp, _fp, _fp, cl, cl, cf, cf, ci, ci, ci]
+        L.pamo_logsumexp_bwd.restype = None; L.pamo_layer_norm_bwd.restype = None
         L.pamo_adam_step.argtypes = [_fp, _fp, _fp, _fp, ctypes.c_size_t, cf, cf, cf, cf, cf, cf, ci, cf, cf]
         L.pamo_adam_step.restype = None
         for name in ("pamo_softmax_fwd", "pamo_softmax_bwd", "pamo_logsumexp_fwd", "pamo_row_mean_fwd",
@@ -269,3 +272,24 @@ def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, d
     lib().pamo_adam_step(_p(p), _p(g), _p(m), _p(v), p.size, f(beta1), f(one_minus_beta1), f(beta2), f(one_minus_beta2),
                          f(eps), f(decay or 0.0), int(bool(decay)), f(step_size), _off(offset))
     return p, m, v
+
+
+def logsumexp_bwd(x, grad, shift, offset=None, approx=(False, False, False), log_softmax=False):
+    """dx of logsumexp over the last dim (grad per row) or of log_softmax (grad per element)."""
+    x2, shape = _rows(x)
+    g = _f32(grad).reshape(x2.shape if log_softmax else (x2.shape[0],))
+    dx = np.empty_like(x2)
+    lib().pamo_logsumexp_bwd(_p(x2), _p(g), float(shift), _p(dx), x2.shape[0], x2.shape[1], int(log_softmax), _off(offset),
+                             int(approx[0]), int(approx[1]), int(approx[2]))
+    return dx.reshape(shape)
+
+
+def layer_norm_bwd(x, weight, grad, eps=1e-5, offset=None, approx=(False, False, False)):
+    """Returns (dx, dw_terms or None): dw_terms[rows, n] sums over rows to the weight gradient."""
+    x2, shape = _rows(x); g, _ = _rows(grad)
+    w = None if weight is None else _f32(weight).ravel()
+    dx = np.empty_like(x2); dw = np.empty_like(x2) if w is not None else None
+    lib().pamo_layer_norm_bwd(_p(x2), None if w is None else _p(w), _p(g), _p(dx), None if dw is None else _p(dw),
+                              x2.shape[0], x2.shape[1], float(np.float32(eps)), _off(offset),
+                              int(approx[0]), int(approx[1]), int(approx[2]))
+    return dx.reshape(shape), dw

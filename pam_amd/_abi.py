@@ -50,7 +50,9 @@ _SIGNATURES = {
     "pam_hip_rowop_workspace_bytes": ([], _z),
     "pam_hip_softmax_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_softmax_bwd": ([_p, _p, _p, _p, _p, _l, _l, _f, _i, _i, _i, _p], _i),
-    "pam_hip_logsumexp_fwd": ([_p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_logsumexp_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_logsumexp_bwd": ([_p, _p, _p, _p, _l, _l, _i, _f, _i, _i, _i, _p], _i),
+    "pam_hip_layer_norm_bwd": ([_p, _p, _p, _p, _p, _l, _l, _f, _f, _i, _i, _i, _p], _i),
     "pam_hip_row_mean_fwd": ([_p, _p, _l, _l, _f, _p], _i),
     "pam_hip_layer_norm_fwd": ([_p, _p, _p, _p, _l, _l, _f, _f, _p], _i),
 }
@@ -309,15 +311,46 @@ class HipRowKernels:
         return dX
 
     def logsumexp_fwd(self, X, offset, want_lse=True, want_log_softmax=False):
+        """Returns (lse or None, log_softmax or None, shift)."""
         rows, n = self._rows("logsumexp_fwd", X)
         lse = torch.empty(rows, dtype=torch.float32, device=X.device) if want_lse else None
         Y = torch.empty_like(X) if want_log_softmax else None
+        shift = torch.empty(1, dtype=torch.float32, device=X.device)
         if X.numel():
             with torch.cuda.device(X.device):
                 ws, nbytes = self._workspace(X.device)
                 _call("pam_hip_logsumexp_fwd", X.data_ptr(), lse.data_ptr() if want_lse else None,
-                      Y.data_ptr() if want_log_softmax else None, rows, n, float(offset), ws.data_ptr(), nbytes, _stream())
-        return lse, Y
+                      Y.data_ptr() if want_log_softmax else None, shift.data_ptr(), rows, n, float(offset),
+                      ws.data_ptr(), nbytes, _stream())
+        return lse, Y, shift
+
+    max_grad_row = 1024          # the gradient kernels keep a row in registers
+
+    def logsumexp_bwd(self, X, grad, shift, offset, approx_a, approx_b, approx_exp, log_softmax):
+        rows, n = self._rows("logsumexp_bwd", X, grad, shift)
+        if grad.numel() != (X.numel() if log_softmax else rows):
+            raise ValueError("logsumexp_bwd: gradient has the wrong size")
+        dX = torch.empty_like(X)
+        if X.numel():
+            with torch.cuda.device(X.device):
+                _call("pam_hip_logsumexp_bwd", X.data_ptr(), grad.data_ptr(), shift.data_ptr(), dX.data_ptr(), rows, n,
+                      int(bool(log_softmax)), float(offset), int(bool(approx_a)), int(bool(approx_b)), int(bool(approx_exp)),
+                      _stream())
+        return dX
+
+    def layer_norm_bwd(self, X, weight, dY, eps, offset, approx_a, approx_b, approx_exp, want_weight_terms):
+        """Returns (dX, per-element weight-gradient terms or None)."""
+        rows, n = self._rows("layer_norm_bwd", X, weight, dY)
+        if dY.shape != X.shape or (weight is not None and weight.numel() != n):
+            raise ValueError("layer_norm_bwd: operand shapes do not match")
+        dX = torch.empty_like(X)
+        terms = torch.empty_like(X) if (want_weight_terms and weight is not None) else None
+        if X.numel():
+            with torch.cuda.device(X.device):
+                _call("pam_hip_layer_norm_bwd", X.data_ptr(), None if weight is None else weight.data_ptr(), dY.data_ptr(),
+                      dX.data_ptr(), None if terms is None else terms.data_ptr(), rows, n, float(eps), float(offset),
+                      int(bool(approx_a)), int(bool(approx_b)), int(bool(approx_exp)), _stream())
+        return dX, terms
 
     def row_mean_fwd(self, X, offset):
         rows, n = self._rows("row_mean_fwd", X)

@@ -5,8 +5,9 @@ additions, subtractions, maxima and sums are ordinary fp32 torch operations, as 
 reference.  Same names and keyword arguments.
 
 Reductions over the last dimension of a contiguous GPU tensor take the single-kernel path of
-`pam_amd.fused` (softmax always, the others when no autograd graph is recorded); every other
-call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
+`pam_amd.fused` (softmax always; logsumexp, log_softmax and layer_norm always for rows of up to
+1024 values, whose gradients are single kernels too, and otherwise, like mean, when no autograd
+graph is recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
 the single-kernel path off.  conv2d on GPU tensors runs on the matrix kernel with the image
 patches read in place instead of unfolded (`implicit_conv = False` switches that off).
 """
@@ -25,11 +26,12 @@ fused_rows = True
 implicit_conv = True
 
 
-def _fused(x, dim, use_kernel, *grad_sources):
-    """True when the call can run as one kernel; grad_sources empty means a gradient is available."""
+def _fused(x, dim, use_kernel, *grad_sources, kernel_gradient=True):
+    """True when the call can run as one kernel: always if that kernel has its gradient, else only
+    when none of grad_sources asks for one."""
     if not (fused_rows and use_kernel and fused.fusable(x, dim)):
         return False
-    return not grad_sources or fused.can_skip_graph(*grad_sources)
+    return kernel_gradient or not fused.needs_graph(*grad_sources)
 
 
 def _pam_kwargs(offset, approx_bwd, use_kernel):
@@ -42,7 +44,7 @@ def mean(input, dim=None, keepdim=False, *, dtype=None, offset=None, approx_bwd=
         dim = tuple(range(input.dim()))
     elif isinstance(dim, int):
         dim = (dim,)
-    if dtype in (None, torch.float32) and _fused(input, dim, use_kernel, input):
+    if dtype in (None, torch.float32) and _fused(input, dim, use_kernel, input, kernel_gradient=False):
         return fused.mean_last(input, keepdim, offset)
     count = math.prod(input.shape[d] for d in dim)
     total = torch.sum(input, dim=dim, keepdim=keepdim, dtype=dtype)
@@ -75,8 +77,8 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
     """pam/pam_ops.py:331-342; inputs must be finite."""
     kw = _pam_kwargs(offset, approx_bwd, use_kernel)
     assert x.isfinite().all()
-    if _fused(x, dim, use_kernel, x):
-        return fused.logsumexp(x, keepdim, offset)
+    if _fused(x, dim, use_kernel, x, kernel_gradient=fused.has_gradient_kernel(x)):
+        return fused.logsumexp(x, keepdim, offset, approx_bwd)
     weights, shift = _scaled_exp2(x, kw, None)
     total = torch.sum(weights, dim=dim, keepdim=keepdim)
     return div(shift + log2(total, **kw), _LOG2_E, **kw)
@@ -84,9 +86,9 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
 
 def log_softmax(x, dim=None, *, offset=None, approx_bwd=False, use_kernel=True):
     """pam/pam_ops.py:345-347"""
-    if _fused(x, dim, use_kernel, x):
+    if _fused(x, dim, use_kernel, x, kernel_gradient=fused.has_gradient_kernel(x)):
         assert x.isfinite().all()
-        return fused.log_softmax(x, offset)
+        return fused.log_softmax(x, offset, approx_bwd)
     return x - logsumexp(x, dim=dim, keepdim=True, **_pam_kwargs(offset, approx_bwd, use_kernel))
 
 
@@ -98,9 +100,9 @@ def layer_norm(x, normalized_shape, weight=None, bias=None, eps=1e-05, *,
     if isinstance(normalized_shape, int):
         normalized_shape = (normalized_shape,)
     assert x.shape[-len(normalized_shape):] == normalized_shape
-    if _fused(x, -1, use_kernel, x, weight, bias) and all(
+    if _fused(x, -1, use_kernel, x, weight, bias, kernel_gradient=math.prod(normalized_shape) <= 1024) and all(
             t is None or (t.is_cuda and t.dtype == torch.float32) for t in (weight, bias)):
-        return fused.layer_norm(x, math.prod(normalized_shape), weight, bias, eps, offset)
+        return fused.layer_norm(x, math.prod(normalized_shape), weight, bias, eps, offset, approx_bwd)
     rows = x.reshape((-1, math.prod(normalized_shape)))
     centred = rows - mean(rows, dim=-1, keepdim=True, **kw)
     variance = mean(mul(centred, centred, **kw), dim=-1, keepdim=True, **kw)

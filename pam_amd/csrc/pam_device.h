@@ -229,6 +229,13 @@ __device__ __forceinline__ float log2_entry(float v, float off, bool has_off)
 __device__ __forceinline__ float pow_half(float v, float off, bool has_off)
 { return v == 0.0f ? 0.0f : exp2_entry(pam_mul_off(log2_entry(v, off, has_off), 0.5f, off, has_off), off, has_off); }
 
+// Exact gradients of the base-2 exp / log entry points as the reference's kernels compute them
+// (pam/cuda_kernels.cu:386-391, 481-484 with log2 2 = 1).
+__device__ __forceinline__ float exp2_entry_bwd(float x, float dy, float off, bool has_off)
+{ return pam_mul_bwd(x, 1.0f, pa_exp2_bwd(pam_mul_off(x, 1.0f, off, has_off), dy), off, has_off); }
+__device__ __forceinline__ float log2_entry_bwd(float x, float dy, float off, bool has_off)
+{ return pa_log2_bwd(x, pam_mul_bwd(pa_log2_signed(x), pad_div_off(1.0f, 1.0f, off, has_off), dy, 1.0f, false)); }
+
 // ---------------------------------------------------------------- unchecked forms
 // Chains of many primitive calls per element (row kernels, optimizer step) pay a range check
 // and a branch per call when built from the functions above.  The forms below compute the

@@ -349,12 +349,13 @@ __device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shif
 
 template <int CH>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
-                                                            float* __restrict__ y, long rows, long n, Offset o,
-                                                            const float* __restrict__ partial, int partials)
+                                                            float* __restrict__ y, float* __restrict__ shift_out, long rows, long n,
+                                                            Offset o, const float* __restrict__ partial, int partials)
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float shift = fold_shift(partial, partials, lane);
+    if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
         auto weight = [&](long, float v) { return exp2_op(scaled(v, o, false) - shift, o); };
@@ -457,6 +458,134 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     }
 }
 
+// ---------------------------------------------------------------- gradients of logsumexp / log_softmax and layer_norm
+// Autograd's chain over the unfused ops, written out (pam/cuda_bindings.py:43-57, 78-97, 224-239,
+// 262-276 for the formulas; pam/pam_ops.py:331-378 for the ops).  Register-resident rows only
+// (n <= 1024); checked arithmetic.
+struct GradMath {
+    Offset o; Approx ap;
+    __device__ __forceinline__ float mul(float a, float b) const { return pam_mul_off(a, b, o.off, o.has); }
+    __device__ __forceinline__ float div(float a, float b) const { return pad_div_off(a, b, o.off, o.has); }
+    // gradient for the first / second operand of c = a (*) b
+    __device__ __forceinline__ float mul_da(float a, float b, float g) const { return ap.a ? mul(g, b) : pam_mul_bwd(a, b, g, o.off, o.has); }
+    __device__ __forceinline__ float mul_db(float a, float b, float g) const { return ap.b ? mul(g, a) : pam_mul_bwd(b, a, g, o.off, o.has); }
+    // gradient for the first / second operand of c = a (/) b
+    __device__ __forceinline__ float div_da(float a, float b, float g) const
+    { const float inv = div(1.0f, b); return ap.a ? mul(inv, g) : pam_mul_bwd(a, inv, g, 1.0f, false); }
+    __device__ __forceinline__ float div_db(float a, float b, float g) const
+    { return ap.b ? -mul(div(div(a, b), b), g) : pad_div_bwd(a, b, g, o.off, o.has); }
+    __device__ __forceinline__ float exp2_dx(float x, float g) const
+    { return ap.e ? mul(mul(exp2_entry(x, o.off, o.has), kLn2), g) : exp2_entry_bwd(x, g, o.off, o.has); }
+    __device__ __forceinline__ float log2_dx(float x, float g) const
+    { return ap.e ? div(div(g, x), kLn2) : log2_entry_bwd(x, g, o.off, o.has); }
+};
+
+// dx of out = logsumexp(x) (per row, gradient g_out) or of y = x - logsumexp(x) (gradient gy per element)
+template <int CH>
+__global__ __launch_bounds__(kThreads) void logsumexp_bwd_kernel(const float* __restrict__ x, const float* __restrict__ grad,
+                                                                const float* __restrict__ shift_in, float* __restrict__ dx,
+                                                                long rows, long n, int log_softmax, Offset o, Approx ap)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float shift = *shift_in;
+    const GradMath m{o, ap};
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n;
+        float xv[CH], gy[CH];
+        load_row<CH>(xv, xr, n, lane, 0.0f);
+        float p = 0.0f, q = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const bool inside = lane + 64L * c < n;
+            gy[c] = (log_softmax && inside) ? grad[r * n + lane + 64L * c] : 0.0f;
+            if (inside) { p = p + exp2_entry(m.mul(xv[c], kLog2E) - shift, o.off, o.has); q = q + gy[c]; }
+        }
+        const float total = wave_sum(p);
+        const float g_out = log_softmax ? -wave_sum(q) : grad[r];       // x - lse: the broadcast lse collects -sum(gy)
+        const float u = shift + log2_entry(total, o.off, o.has);
+        const float du = m.div_da(u, kLog2E, g_out);
+        const float dtotal = m.log2_dx(total, du);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const long i = lane + 64L * c;
+            if (i < n) {
+                const float t = m.mul(xv[c], kLog2E) - shift;
+                const float d = m.mul_da(xv[c], kLog2E, m.exp2_dx(t, dtotal));
+                dx[r * n + i] = log_softmax ? gy[c] + d : d;
+            }
+        }
+    }
+}
+
+// dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias
+template <int CH>
+__global__ __launch_bounds__(kThreads) void layer_norm_bwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                                 const float* __restrict__ gy, float* __restrict__ dx,
+                                                                 float* __restrict__ dw_terms, long rows, long n, float eps,
+                                                                 Offset o, Approx ap)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float count = (float)n;
+    const GradMath m{o, ap};
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* xr = x + r * n; const float* gr = gy + r * n;
+        float cen[CH], g[CH];
+        load_row<CH>(cen, xr, n, lane, 0.0f);
+        load_row<CH>(g, gr, n, lane, 0.0f);
+        // forward values
+        float p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) p = p + cen[c];
+        const float s1 = wave_sum(p);
+        const float mu = m.div(s1, count);
+        p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) { cen[c] = cen[c] - mu; if (lane + 64L * c < n) p = p + m.mul(cen[c], cen[c]); }
+        const float s2 = wave_sum(p);
+        const float v = m.div(s2, count) + eps;
+        const float lg = log2_entry(v, o.off, o.has);
+        const float half = m.mul(lg, 0.5f);
+        const float denom = v == 0.0f ? 0.0f : exp2_entry(half, o.off, o.has);
+        // through the weight product and the quotient; the row sum for the broadcast denominator
+        p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const long i = lane + 64L * c;
+            if (i < n) {
+                if (weight) {
+                    const float xn = m.div(cen[c], denom), wi = weight[i];
+                    if (dw_terms) dw_terms[r * n + i] = m.mul_db(xn, wi, g[c]);
+                    g[c] = m.mul_da(xn, wi, g[c]);
+                }
+                p = p + m.div_db(cen[c], denom, g[c]);
+            }
+        }
+        float d = wave_sum(p);
+        if (v == 0.0f) d = 0.0f;                                   // where(v == 0, 0, exp2(..))
+        d = m.exp2_dx(half, d);
+        d = m.mul_da(lg, 0.5f, d);
+        d = m.log2_dx(v, d);                                       // = d var
+        const float ds2 = m.div_da(s2, count, d);
+        // gradients reaching the centred values: quotient, then the two operands of c (*) c
+        p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            if (lane + 64L * c < n) {
+                float dc = m.div_da(cen[c], denom, g[c]);
+                dc = dc + m.mul_da(cen[c], cen[c], ds2);
+                dc = dc + m.mul_db(cen[c], cen[c], ds2);
+                g[c] = dc;
+                p = p + dc;
+            }
+        }
+        const float ds1 = m.div_da(s1, count, -wave_sum(p));       // mu is subtracted: it collects -sum(dc)
+#pragma unroll
+        for (int c = 0; c < CH; ++c) { const long i = lane + 64L * c; if (i < n) dx[r * n + i] = g[c] + ds1; }
+    }
+}
+
 // smallest register-resident variant that holds a row of n values, 0 for the streaming one
 int row_chunks(long n)
 {
@@ -472,6 +601,15 @@ int row_chunks(long n)
     case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 16: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     default: hipLaunchKernelGGL(KERNEL<0>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                    \
+    }
+
+#define PAM_ROW_DISPATCH_REGS(KERNEL, n, grid, st, ...)                                                         \
+    switch (row_chunks(n)) {                                                                                    \
+    case 1: hipLaunchKernelGGL(KERNEL<1>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 2: hipLaunchKernelGGL(KERNEL<2>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 4: hipLaunchKernelGGL(KERNEL<4>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    default: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     }
 
 int g_cus = 0;
@@ -550,7 +688,7 @@ int pam_hip_softmax_bwd(const float* x, const float* dy, const float* row_sum, c
     return pamhost::check_launch("softmax_bwd");
 }
 
-int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, long rows, long n, float offset,
+int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, float* shift, long rows, long n, float offset,
                           void* workspace, size_t workspace_bytes, void* stream)
 {
     int rc = check_rows("logsumexp_fwd", rows, n);
@@ -560,7 +698,7 @@ int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, long r
     hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
     rc = launch_max("logsumexp_fwd", x, rows, n, o, 0, workspace, workspace_bytes, st, &partials);
     if (rc != PAM_HIP_OK) return rc;
-    PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows)), st, x, lse, log_softmax, rows, n, o,
+    PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows)), st, x, lse, log_softmax, shift, rows, n, o,
                      (const float*)workspace, partials);
     return pamhost::check_launch("logsumexp_fwd");
 }
@@ -586,6 +724,34 @@ int pam_hip_layer_norm_fwd(const float* x, const float* weight, const float* bia
     const Offset o{offset, offset != 1.0f};
     PAM_ROW_DISPATCH(layer_norm_fwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, bias, y, rows, n, eps, o);
     return pamhost::check_launch("layer_norm_fwd");
+}
+
+int pam_hip_logsumexp_bwd(const float* x, const float* grad, const float* shift, float* dx, long rows, long n,
+                          int log_softmax, float offset, int approx_a, int approx_b, int approx_exp, void* stream)
+{
+    int rc = check_rows("logsumexp_bwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0 || n == 0) return PAM_HIP_OK;
+    if (!x || !grad || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_bwd: null pointer");
+    if (n > 1024) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_bwd: rows of at most 1024 values");
+    Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
+    PAM_ROW_DISPATCH_REGS(logsumexp_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n,
+                          log_softmax, o, ap);
+    return pamhost::check_launch("logsumexp_bwd");
+}
+
+int pam_hip_layer_norm_bwd(const float* x, const float* weight, const float* dy, float* dx, float* dw_terms, long rows, long n,
+                           float eps, float offset, int approx_a, int approx_b, int approx_exp, void* stream)
+{
+    int rc = check_rows("layer_norm_bwd", rows, n);
+    if (rc != PAM_HIP_OK) return rc;
+    if (rows == 0 || n == 0) return PAM_HIP_OK;
+    if (!x || !dy || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_bwd: null pointer");
+    if (n > 1024) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_bwd: rows of at most 1024 values");
+    Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
+    PAM_ROW_DISPATCH_REGS(layer_norm_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms,
+                          rows, n, eps, o, ap);
+    return pamhost::check_launch("layer_norm_bwd");
 }
 
 }  // extern "C"

@@ -52,12 +52,8 @@ class softmax_autograd(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad):
         rows, row_sum, shift = ctx.saved_tensors
-        approx_a, approx_b = _both(ctx.approx_bwd)
-        # exp2's backward tests the flag's truth value, so a pair counts as set
-        # (pam/cuda_bindings.py:227)
-        approx_exp = bool(ctx.approx_bwd)
         g = grad.contiguous().view(rows.shape)
-        dx = row_kernels.softmax_bwd(rows, g, row_sum, shift, ctx.offset, approx_a, approx_b, approx_exp)
+        dx = row_kernels.softmax_bwd(rows, g, row_sum, shift, ctx.offset, *_flags(ctx.approx_bwd))
         return dx.view(grad.shape), None, None
 
 
@@ -65,22 +61,52 @@ def softmax(x, offset=None, approx_bwd=False):
     return softmax_autograd.apply(x, offset, approx_bwd)
 
 
-# The remaining fused forwards have no fused gradient: they serve calls that record no
-# graph, and `composites` keeps the unfused chain for calls that do.
-
-def can_skip_graph(*tensors):
-    return not _wants_grad(*tensors)
-
-
-def logsumexp(x, keepdim, offset=None):
-    lse, _ = row_kernels.logsumexp_fwd(x.reshape(-1, x.shape[-1]), _offset_value(offset), True, False)
-    shape = x.shape[:-1] + ((1,) if keepdim else ())
-    return lse.view(shape)
+def _flags(approx_bwd):
+    """(first operands, second operands, exp / log): the last tests the flag's truth value, so a
+    pair counts as set (pam/cuda_bindings.py:227, 267)."""
+    a, b = _both(approx_bwd)
+    return a, b, bool(approx_bwd)
 
 
-def log_softmax(x, offset=None):
-    _, y = row_kernels.logsumexp_fwd(x.reshape(-1, x.shape[-1]), _offset_value(offset), False, True)
-    return y.view(x.shape)
+def has_gradient_kernel(x):
+    """The gradient kernels of logsumexp, log_softmax and layer_norm keep a row in registers."""
+    return x.shape[-1] <= row_kernels.max_grad_row
+
+
+def needs_graph(*tensors):
+    return _wants_grad(*tensors)
+
+
+class logsumexp_autograd(torch.autograd.Function):
+    """logsumexp (as_log_softmax False) or log_softmax = x - logsumexp(x) over the last dimension."""
+
+    @staticmethod
+    def forward(ctx, x, offset, approx_bwd, as_log_softmax, keepdim):
+        ctx.offset = _offset_value(offset)
+        ctx.approx_bwd = approx_bwd
+        ctx.as_log_softmax = as_log_softmax
+        rows = x.reshape(-1, x.shape[-1])
+        lse, y, shift = row_kernels.logsumexp_fwd(rows, ctx.offset, not as_log_softmax, as_log_softmax)
+        ctx.save_for_backward(rows, shift)
+        if as_log_softmax:
+            return y.view(x.shape)
+        return lse.view(x.shape[:-1] + ((1,) if keepdim else ()))
+
+    @staticmethod
+    def backward(ctx, grad):
+        rows, shift = ctx.saved_tensors
+        g = grad.contiguous().view(rows.shape if ctx.as_log_softmax else (rows.shape[0],))
+        dx = row_kernels.logsumexp_bwd(rows, g, shift, ctx.offset, *_flags(ctx.approx_bwd), ctx.as_log_softmax)
+        return dx, None, None, None, None
+
+
+def logsumexp(x, keepdim, offset=None, approx_bwd=False):
+    out = logsumexp_autograd.apply(x.reshape(-1, x.shape[-1]), offset, approx_bwd, False, True)
+    return out.view(x.shape[:-1] + ((1,) if keepdim else ()))
+
+
+def log_softmax(x, offset=None, approx_bwd=False):
+    return logsumexp_autograd.apply(x.reshape(-1, x.shape[-1]), offset, approx_bwd, True, True).view(x.shape)
 
 
 def mean_last(x, keepdim, offset=None):
@@ -88,10 +114,37 @@ def mean_last(x, keepdim, offset=None):
     return y.view(x.shape[:-1] + ((1,) if keepdim else ()))
 
 
-def layer_norm(x, n, weight, bias, eps, offset=None):
-    w = None if weight is None else weight.detach().contiguous().view(-1)
-    b = None if bias is None else bias.detach().contiguous().view(-1)
-    return row_kernels.layer_norm_fwd(x.reshape(-1, n), w, b, eps, _offset_value(offset)).view(x.shape)
+class layer_norm_autograd(torch.autograd.Function):
+    """layer_norm over the last n values of each row; weight and bias of n values or None."""
+
+    @staticmethod
+    def forward(ctx, rows, weight, bias, eps, offset, approx_bwd):
+        ctx.offset = _offset_value(offset)
+        ctx.approx_bwd = approx_bwd
+        ctx.eps = eps
+        ctx.has_bias = bias is not None
+        w = None if weight is None else weight.contiguous().view(-1)
+        b = None if bias is None else bias.contiguous().view(-1)
+        ctx.save_for_backward(rows, w)
+        return row_kernels.layer_norm_fwd(rows, w, b, eps, ctx.offset)
+
+    @staticmethod
+    def backward(ctx, grad):
+        rows, w = ctx.saved_tensors
+        g = grad.contiguous()
+        want_w = w is not None and ctx.needs_input_grad[1]
+        dx, terms = row_kernels.layer_norm_bwd(rows, w, g, ctx.eps, ctx.offset, *_flags(ctx.approx_bwd), want_w)
+        # the broadcast weight and bias collect their gradients by a sum over the rows, as autograd's expand does
+        dw = terms.sum(0) if want_w else None
+        db = g.sum(0) if (ctx.has_bias and ctx.needs_input_grad[2]) else None
+        return dx, dw, db, None, None, None
+
+
+def layer_norm(x, n, weight, bias, eps, offset=None, approx_bwd=False):
+    w = None if weight is None else weight.reshape(-1)
+    b = None if bias is None else bias.reshape(-1)
+    out = layer_norm_autograd.apply(x.reshape(-1, n), w, b, eps, offset, approx_bwd)
+    return out.view(x.shape)
 
 
 # ---------------------------------------------------------------- convolution on image patches read in place

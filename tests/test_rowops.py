@@ -190,6 +190,44 @@ def test_softmax_gradient_chain_is_what_autograd_does(on_cpu, approx):
         assert (got[np.isneginf(x)] == 0).all()
 
 
+def _flags(approx):
+    return (approx, approx, approx) if isinstance(approx, bool) else (approx[0], approx[1], True)
+
+
+@pytest.mark.parametrize("approx", [False, True, (True, False), (False, True)])
+def test_logsumexp_and_layer_norm_gradient_chains_are_what_autograd_does(on_cpu, approx):
+    """The oracle's gradient restatements against torch autograd over the unfused compositions
+    (oracle-backed kernel object, CPU): same formulas, torch's summation order."""
+    o = on_cpu
+    x = rows_case(31, 6, 40, masks=False)
+    rng = np.random.RandomState(32)
+    g_rows = rng.standard_normal(6).astype(np.float32); g_full = rng.standard_normal(x.shape).astype(np.float32)
+    w = (rng.standard_normal(40) + 2).astype(np.float32); b = rng.standard_normal(40).astype(np.float32)
+
+    def close(got, want, tol=1e-5):
+        scale = np.abs(want).max()
+        assert np.isfinite(want).all() and np.abs(got - want).max() <= tol * scale, (np.abs(got - want).max(), scale)
+
+    for off in (None, OFF):
+        shift = np.floor(o.pam(x, C, off).max())
+        xt = torch.from_numpy(x.copy()).requires_grad_()
+        composites.logsumexp(xt, dim=-1, offset=off, approx_bwd=approx).backward(torch.from_numpy(g_rows))
+        close(o.logsumexp_bwd(x, g_rows, shift, off, _flags(approx)), xt.grad.numpy())
+        xt = torch.from_numpy(x.copy()).requires_grad_()
+        composites.log_softmax(xt, dim=-1, offset=off, approx_bwd=approx).backward(torch.from_numpy(g_full))
+        close(o.logsumexp_bwd(x, g_full, shift, off, _flags(approx), log_softmax=True), xt.grad.numpy())
+        for ww, bb in [(None, None), (w, b)]:
+            xt = torch.from_numpy(x.copy()).requires_grad_()
+            wt = None if ww is None else torch.from_numpy(ww.copy()).requires_grad_()
+            bt = None if bb is None else torch.from_numpy(bb.copy()).requires_grad_()
+            composites.layer_norm(xt, 40, wt, bt, offset=off, approx_bwd=approx).backward(torch.from_numpy(g_full))
+            dx, terms = o.layer_norm_bwd(x, ww, g_full, 1e-5, off, _flags(approx))
+            close(dx, xt.grad.numpy(), 2e-5)
+            if ww is not None:
+                close(terms.sum(0), wt.grad.numpy())
+                close(g_full.sum(0), bt.grad.numpy())
+
+
 # ------------------------------------------------------------------ GPU: HIP kernels == oracle fused
 def _dev(a):
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
@@ -207,7 +245,7 @@ def test_gpu_softmax_forward_backward(oracle, off):
             y = pam_amd.softmax(xt, dim=-1, offset=off, approx_bwd=approx)
             assert_same_bits(y.detach().cpu().numpy(), want, f"softmax {rows}x{n}")
             y.backward(_dev(g))
-            flags = (approx, approx, approx) if isinstance(approx, bool) else (approx[0], approx[1], True)
+            flags = _flags(approx)
             assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, off, flags),
                              f"softmax gradient {rows}x{n} approx={approx}")
 
@@ -296,3 +334,64 @@ def test_gpu_attention_softmax_full_size(oracle):
     assert_same_bits(y.detach().cpu().numpy(), want, "softmax 192x197x197")
     assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, None, (True, True, True)), "its gradient")
     assert np.abs(want.sum(-1) - 1).max() < 0.1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("off", [None, OFF])
+def test_gpu_logsumexp_and_layer_norm_gradients(oracle, off):
+    for rows, n in [(1, 1), (3, 7), (5, 64), (40, 192), (9, 513), (6, 1024)]:
+        x = rows_case(rows * 13 + n, rows, n, masks=False)
+        rng = np.random.RandomState(n)
+        g_rows = rng.standard_normal(rows).astype(np.float32); g_full = rng.standard_normal(x.shape).astype(np.float32)
+        w = (rng.standard_normal(n) + 2).astype(np.float32); b = rng.standard_normal(n).astype(np.float32)
+        shift = np.floor(oracle.pam(x, C, off).max())
+        for approx in (False, True, (True, False)):
+            xt = _dev(x).requires_grad_()
+            pam_amd.logsumexp(xt, dim=-1, offset=off, approx_bwd=approx).backward(_dev(g_rows))
+            assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(x, g_rows, shift, off, _flags(approx)), f"logsumexp gradient {rows}x{n}")
+            xt = _dev(x).requires_grad_()
+            y = pam_amd.log_softmax(xt, dim=-1, offset=off, approx_bwd=approx)
+            assert_same_bits(y.detach().cpu().numpy(), oracle.logsumexp_fwd(x, off, with_log_softmax=True)[1], "log_softmax")
+            y.backward(_dev(g_full))
+            assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(x, g_full, shift, off, _flags(approx), log_softmax=True),
+                             f"log_softmax gradient {rows}x{n}")
+            for ww, bb in [(None, None), (w, b)]:
+                xt = _dev(x).requires_grad_()
+                wt = None if ww is None else _dev(ww).requires_grad_(); bt = None if bb is None else _dev(bb).requires_grad_()
+                y = pam_amd.layer_norm(xt, n, wt, bt, offset=off, approx_bwd=approx)
+                assert_same_bits(y.detach().cpu().numpy(), oracle.layer_norm_fwd(x, ww, bb, 1e-5, off), "layer_norm")
+                y.backward(_dev(g_full))
+                dx, terms = oracle.layer_norm_bwd(x, ww, g_full, 1e-5, off, _flags(approx))
+                assert_same_bits(xt.grad.cpu().numpy(), dx, f"layer_norm gradient {rows}x{n} approx={approx}")
+                if ww is not None:
+                    want_w = torch.from_numpy(terms).sum(0).numpy()
+                    assert np.abs(wt.grad.cpu().numpy() - want_w).max() <= 1e-5 * np.abs(want_w).max() + 1e-7
+                    assert np.allclose(bt.grad.cpu().numpy(), g_full.sum(0), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_gpu_row_gradients_match_unfused_composition():
+    """LayerNorm and log_softmax in training on the GPU: single kernels against the chains of
+    primitive kernels, values and all gradients, up to the order of the sums."""
+    x = rows_case(41, 8 * 25, 96, masks=False).reshape(8, 25, 96)
+    g = np.random.RandomState(5).standard_normal(x.shape).astype(np.float32)
+    res = {}
+    for fused_on in (True, False):
+        composites.fused_rows = fused_on
+        try:
+            torch.manual_seed(0)
+            ln = pam_amd.LayerNorm(96, approx_bwd=True).cuda()
+            with torch.no_grad():
+                ln.weight.copy_(torch.randn(96).cuda() + 2); ln.bias.copy_(torch.randn(96).cuda())
+            xt = _dev(x).requires_grad_()
+            y = pam_amd.log_softmax(ln(xt), dim=-1, approx_bwd=True)
+            y.backward(_dev(g))
+            res[fused_on] = [t.detach().cpu().numpy() for t in (y, xt.grad, ln.weight.grad, ln.bias.grad)]
+        finally:
+            composites.fused_rows = True
+    for a, b in zip(res[True], res[False]):
+        assert np.abs(a - b).max() <= 2e-5 * np.abs(b).max()
+    # rows longer than the gradient kernels hold fall back to the chain when a graph is recorded
+    wide = _dev(rows_case(42, 3, 1500, masks=False)).requires_grad_()
+    pam_amd.log_softmax(wide, dim=-1, approx_bwd=True).sum().backward()
+    assert torch.isfinite(wide.grad).all()
