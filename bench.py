@@ -196,11 +196,25 @@ def main():
                 ("layer_norm_fwd", 8, lambda: R.layer_norm_fwd(xs, wv, bv, 1e-5, 1.0)),
                 ("row_mean_fwd", 4, lambda: R.row_mean_fwd(xs, 1.0)),
             )
+            if c <= R.max_grad_row:
+                row_ops += (
+                    ("layer_norm_bwd_approx", 16, lambda: R.layer_norm_bwd(xs, wv, gs, 1e-5, 1.0, True, True, True, True)),
+                    ("log_softmax_bwd_approx", 12, lambda: R.logsumexp_bwd(xs, gs, sh, 1.0, True, True, True, True)),
+                )
             for name, bpe, fn in row_ops:
                 ms = event_time_ms(fn, 10, torch)
                 other[f"{name}_{tag}"] = {"ms": round(ms, 4), "GBps": round(bpe * r * c / ms / 1e6, 1),
                                           "hbm_frac": round(bpe * r * c / ms / 1e6 / 8000.0, 3)}
             del xs, gs, ys
+        # convolution with the image patches read in place (forward; PAM-MAC/s against the vector peak)
+        for tag, (cb, cc, chh, co_, ck, cs, cp) in {"conv3x3_128x64x32x32_to128": (128, 64, 32, 128, 3, 1, 1),
+                                                     "patch_embed_64x3x224x224_16x16_to192": (64, 3, 224, 192, 16, 16, 0)}.items():
+            xc = torch.randn(cb, cc, chh, chh, generator=g).to(dev); wc = (torch.randn(co_, cc, ck, ck, generator=g) * 0.05).to(dev)
+            ho = (chh + 2 * cp - ck) // cs + 1
+            cm = cb * co_ * ho * ho * cc * ck * ck
+            ms = event_time_ms(lambda: abi.conv2d_fwd(xc, wc, (cs, cs), (cp, cp), 1.0), 10, torch)
+            other[tag] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1), "valu_frac": round(2 * cm / (ms * 1e-3) / lane_peak, 4)}
+            del xc, wc
         na = 1 << 26
         pa, ga, ma, va = (torch.randn(na, generator=g).to(dev) * s_ for s_ in (1.0, 1e-2, 1e-2, 1e-4))
         va.abs_()
