@@ -71,6 +71,11 @@ int pam_hip_pa_log_fwd(const float *x, float *y, size_t n, float base, float off
 /*                                                replaces pa_log_bwd (:488-516) */
 int pam_hip_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, float base, float offset, void *stream);
 
+/* Tuning hook for experiments: forces the k-tile depth (16 or 32; 0 = automatic) and the number of
+ * k chunks (0 = automatic) of the matrix products for the calling process.  No counterpart in the
+ * reference; pam_hip_gemm_plan and pam_hip_gemm_workspace_bytes follow the forced values. */
+void pam_hip_set_tuning(int k_tile, int k_chunks);
+
 /* ---- matrix products (pam/cuda_kernels.cu:574-927) ------------------------------------- */
 /* A matrix operand: pointer, batch stride, row stride, column stride (elements). */
 #define PAM_HIP_MAT(name) const float *name, long name##_sb, long name##_sr, long name##_sc
