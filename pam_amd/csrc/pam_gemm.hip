@@ -318,10 +318,11 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
     for (int t = 0; t < ktiles; ++t) {
         const int cur = t & 1;
         const int k0 = kbegin + t * BK;
-        if (t + 1 < ktiles) {
-            ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid, g.cv);
-            rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid, g.cv);
-        }
+        // The next tile is fetched unconditionally: past the end the clamped addresses re-read the last
+        // tile and the values are dropped.  A conditional fetch would merge with the registers' old
+        // contents and make the compiler wait for the data right here.
+        ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid, g.cv);
+        rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid, g.cv);
         const int kcount = min(BK, kend - k0);
         uint32_t verdict = 0;                     // 0 plain loop, 1 zeros present, 2 guarded
         if (MODE != MODE_STD) {
@@ -397,10 +398,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
                 }
         };
 
-        if (verdict == 1 && MODE == MODE_PAM) {
-#pragma unroll 2
-            for (int kk = 0; kk < kcount; ++kk) zeros_step(kk);
-        } else if (verdict == 0) {
+        if (__builtin_expect(verdict == 0, 1)) {
             if (kcount == BK) {
                 // fragments for step kk+1 are read from LDS while step kk is computed
                 uint32_t fa[2][TM], fb[2][TN];
@@ -422,6 +420,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g,
 #pragma unroll 1
                 for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
             }
+        } else if (verdict == 1 && MODE == MODE_PAM) {
+#pragma unroll 2
+            for (int kk = 0; kk < kcount; ++kk) zeros_step(kk);
         } else {
 #pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) guarded_step(kk);
