@@ -22,6 +22,8 @@ using namespace pamdev;
 
 namespace {
 
+// Wavefronts per SIMD the row kernels are compiled for (a cap of 128 registers per lane); the
+// gradient kernels for the longest register-resident rows take 2 (they would spill otherwise).
 #ifndef PAM_ROW_WAVES
 #define PAM_ROW_WAVES 4
 #endif
@@ -461,128 +463,185 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 // ---------------------------------------------------------------- gradients of logsumexp / log_softmax and layer_norm
 // Autograd's chain over the unfused ops, written out (pam/cuda_bindings.py:43-57, 78-97, 224-239,
 // 262-276 for the formulas; pam/pam_ops.py:331-378 for the ops).  Register-resident rows only
-// (n <= 1024); checked arithmetic.
-struct GradMath {
+// (n <= 1024).  GradChecked serves every combination of exact and approximate gradients;
+// GradUnchecked is the all-approximate chain on the branch-free primitives, tried first and kept
+// when every value it touched was a normal number.
+struct GradChecked {
     Offset o; Approx ap;
-    __device__ __forceinline__ float mul(float a, float b) const { return pam_mul_off(a, b, o.off, o.has); }
-    __device__ __forceinline__ float div(float a, float b) const { return pad_div_off(a, b, o.off, o.has); }
+    __device__ __forceinline__ float mul(float a, float b) { return pam_mul_off(a, b, o.off, o.has); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_div_off(a, b, o.off, o.has); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry(t, o.off, o.has); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry(v, o.off, o.has); }
     // gradient for the first / second operand of c = a (*) b
-    __device__ __forceinline__ float mul_da(float a, float b, float g) const { return ap.a ? mul(g, b) : pam_mul_bwd(a, b, g, o.off, o.has); }
-    __device__ __forceinline__ float mul_db(float a, float b, float g) const { return ap.b ? mul(g, a) : pam_mul_bwd(b, a, g, o.off, o.has); }
+    __device__ __forceinline__ float mul_da(float a, float b, float g) { return ap.a ? mul(g, b) : pam_mul_bwd(a, b, g, o.off, o.has); }
+    __device__ __forceinline__ float mul_db(float a, float b, float g) { return ap.b ? mul(g, a) : pam_mul_bwd(b, a, g, o.off, o.has); }
     // gradient for the first / second operand of c = a (/) b
-    __device__ __forceinline__ float div_da(float a, float b, float g) const
+    __device__ __forceinline__ float div_da(float a, float b, float g)
     { const float inv = div(1.0f, b); return ap.a ? mul(inv, g) : pam_mul_bwd(a, inv, g, 1.0f, false); }
-    __device__ __forceinline__ float div_db(float a, float b, float g) const
+    __device__ __forceinline__ float div_db(float a, float b, float g)
     { return ap.b ? -mul(div(div(a, b), b), g) : pad_div_bwd(a, b, g, o.off, o.has); }
-    __device__ __forceinline__ float exp2_dx(float x, float g) const
-    { return ap.e ? mul(mul(exp2_entry(x, o.off, o.has), kLn2), g) : exp2_entry_bwd(x, g, o.off, o.has); }
-    __device__ __forceinline__ float log2_dx(float x, float g) const
+    __device__ __forceinline__ float exp2_dx(float x, float g)
+    { return ap.e ? mul(mul(exp2(x), kLn2), g) : exp2_entry_bwd(x, g, o.off, o.has); }
+    __device__ __forceinline__ float log2_dx(float x, float g)
     { return ap.e ? div(div(g, x), kLn2) : log2_entry_bwd(x, g, o.off, o.has); }
+    __device__ __forceinline__ bool valid() const { return true; }
 };
+struct GradUnchecked {
+    Offset o; Span sp;
+    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, o.has, sp); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, o.has, sp); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, o.has, sp); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float mul_da(float, float b, float g) { return mul(g, b); }
+    __device__ __forceinline__ float mul_db(float a, float, float g) { return mul(g, a); }
+    __device__ __forceinline__ float div_da(float, float b, float g) { return mul(div(1.0f, b), g); }
+    __device__ __forceinline__ float div_db(float a, float b, float g) { return -mul(div(div(a, b), b), g); }
+    __device__ __forceinline__ float exp2_dx(float x, float g) { return mul(mul(exp2(x), kLn2), g); }
+    __device__ __forceinline__ float log2_dx(float x, float g) { return div(div(g, x), kLn2); }
+    __device__ __forceinline__ bool valid() const { return sp.normal(); }
+};
+
+// One row of the logsumexp / log_softmax gradient.  xv: the inputs (any fill past the end); gy: the
+// per-element gradients (log_softmax) with 1.0 past the end; out: dx.  Lanes past the end of the
+// row work on stand-in values that are never stored or summed.
+template <int CH, class G>
+__device__ __forceinline__ void logsumexp_grad_row(const float (&xv)[CH], const float (&gy)[CH], float (&out)[CH], float g_row,
+                                                   bool log_softmax, float shift, int lane, long n, G& m)
+{
+    float p = 0.0f, q = 0.0f, t[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool inside = lane + 64L * c < n;
+        const float s = m.mul(inside ? xv[c] : 1.0f, kLog2E) - shift;
+        t[c] = inside ? s : 0.5f;
+        const float e = m.exp2(t[c]);
+        if (inside) { p = p + e; q = q + gy[c]; }
+    }
+    const float total = wave_sum(p);
+    const float g_out = log_softmax ? -wave_sum(q) : g_row;         // x - lse: the broadcast lse collects -sum(gy)
+    const float u = shift + m.log2(total);
+    const float du = m.div_da(u, kLog2E, g_out);
+    const float dtotal = m.log2_dx(total, du);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool inside = lane + 64L * c < n;
+        const float d = m.mul_da(inside ? xv[c] : 1.0f, kLog2E, m.exp2_dx(t[c], dtotal));
+        out[c] = log_softmax ? gy[c] + d : d;
+    }
+}
 
 // dx of out = logsumexp(x) (per row, gradient g_out) or of y = x - logsumexp(x) (gradient gy per element)
 template <int CH>
-__global__ __launch_bounds__(kThreads) void logsumexp_bwd_kernel(const float* __restrict__ x, const float* __restrict__ grad,
-                                                                const float* __restrict__ shift_in, float* __restrict__ dx,
-                                                                long rows, long n, int log_softmax, Offset o, Approx ap)
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(CH >= 16 ? 2 : PAM_ROW_WAVES))) void logsumexp_bwd_kernel(
+    const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
+    long rows, long n, int log_softmax, Offset o, Approx ap)
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float shift = *shift_in;
-    const GradMath m{o, ap};
     for (long r = wave; r < rows; r += nwaves) {
-        const float* xr = x + r * n;
-        float xv[CH], gy[CH];
-        load_row<CH>(xv, xr, n, lane, 0.0f);
-        float p = 0.0f, q = 0.0f;
+        float xv[CH], gy[CH], out[CH];
+        load_row<CH>(xv, x + r * n, n, lane, 0.0f);
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const bool inside = lane + 64L * c < n;
-            gy[c] = (log_softmax && inside) ? grad[r * n + lane + 64L * c] : 0.0f;
-            if (inside) { p = p + exp2_entry(m.mul(xv[c], kLog2E) - shift, o.off, o.has); q = q + gy[c]; }
+        for (int c = 0; c < CH; ++c) gy[c] = 1.0f;
+        if (log_softmax) load_row<CH>(gy, grad + r * n, n, lane, 1.0f);
+        const float g_row = log_softmax ? 0.0f : grad[r];
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            GradUnchecked u{o};
+            logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lane, n, u);
+            done = __ballot(!u.valid()) == 0ull;
         }
-        const float total = wave_sum(p);
-        const float g_out = log_softmax ? -wave_sum(q) : grad[r];       // x - lse: the broadcast lse collects -sum(gy)
-        const float u = shift + log2_entry(total, o.off, o.has);
-        const float du = m.div_da(u, kLog2E, g_out);
-        const float dtotal = m.log2_dx(total, du);
+        if (!done) { GradChecked k{o, ap}; logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lane, n, k); }
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const long i = lane + 64L * c;
-            if (i < n) {
-                const float t = m.mul(xv[c], kLog2E) - shift;
-                const float d = m.mul_da(xv[c], kLog2E, m.exp2_dx(t, dtotal));
-                dx[r * n + i] = log_softmax ? gy[c] + d : d;
-            }
-        }
+        for (int c = 0; c < CH; ++c) { const long i = lane + 64L * c; if (i < n) dx[r * n + i] = out[c]; }
     }
+}
+
+// One row of the layer_norm gradient.  cen: x on entry, overwritten; g: dy on entry (1.0 past the
+// end), dx on exit; terms: the per-element terms of the weight gradient (if weight).
+template <int CH, class G>
+__device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)[CH], float (&terms)[CH],
+                                                    const float* __restrict__ weight, int lane, long n, float count, float eps, G& m)
+{
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) p = p + cen[c];                        // the fill adds +0
+    const float s1 = wave_sum(p);
+    const float mu = m.div(s1, count);
+    p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) { cen[c] = cen[c] - mu; const float sq = m.mul(cen[c], cen[c]); if (lane + 64L * c < n) p = p + sq; }
+    const float s2 = wave_sum(p);
+    const float v = m.div(s2, count) + eps;
+    const float lg = m.log2(v);
+    const float half = m.mul(lg, 0.5f);
+    const float root = m.exp2(half);
+    const float denom = v == 0.0f ? 0.0f : root;
+    // through the weight product and the quotient; the row sum for the broadcast denominator
+    p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const long i = lane + 64L * c; const bool inside = i < n;
+        if (weight) {
+            const float xn = m.div(cen[c], denom), wi = inside ? weight[i] : 1.0f;
+            terms[c] = m.mul_db(xn, wi, g[c]);
+            g[c] = m.mul_da(xn, wi, g[c]);
+        }
+        const float d = m.div_db(cen[c], denom, g[c]);
+        if (inside) p = p + d;
+    }
+    float d = wave_sum(p);
+    if (v == 0.0f) d = 0.0f;                                            // where(v == 0, 0, exp2(..))
+    d = m.exp2_dx(half, d);
+    d = m.mul_da(lg, 0.5f, d);
+    d = m.log2_dx(v, d);                                                // = d var
+    const float ds2 = m.div_da(s2, count, d);
+    // gradients reaching the centred values: quotient, then the two operands of c (*) c
+    p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        float dc = m.div_da(cen[c], denom, g[c]);
+        dc = dc + m.mul_da(cen[c], cen[c], ds2);
+        dc = dc + m.mul_db(cen[c], cen[c], ds2);
+        g[c] = dc;
+        if (lane + 64L * c < n) p = p + dc;
+    }
+    const float ds1 = m.div_da(s1, count, -wave_sum(p));                // mu is subtracted: it collects -sum(dc)
+#pragma unroll
+    for (int c = 0; c < CH; ++c) g[c] = g[c] + ds1;
 }
 
 // dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias
 template <int CH>
-__global__ __launch_bounds__(kThreads) void layer_norm_bwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
-                                                                 const float* __restrict__ gy, float* __restrict__ dx,
-                                                                 float* __restrict__ dw_terms, long rows, long n, float eps,
-                                                                 Offset o, Approx ap)
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(CH >= 16 ? 2 : PAM_ROW_WAVES))) void layer_norm_bwd_kernel(
+    const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
+    float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float count = (float)n;
-    const GradMath m{o, ap};
     for (long r = wave; r < rows; r += nwaves) {
-        const float* xr = x + r * n; const float* gr = gy + r * n;
-        float cen[CH], g[CH];
-        load_row<CH>(cen, xr, n, lane, 0.0f);
-        load_row<CH>(g, gr, n, lane, 0.0f);
-        // forward values
-        float p = 0.0f;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) p = p + cen[c];
-        const float s1 = wave_sum(p);
-        const float mu = m.div(s1, count);
-        p = 0.0f;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) { cen[c] = cen[c] - mu; if (lane + 64L * c < n) p = p + m.mul(cen[c], cen[c]); }
-        const float s2 = wave_sum(p);
-        const float v = m.div(s2, count) + eps;
-        const float lg = log2_entry(v, o.off, o.has);
-        const float half = m.mul(lg, 0.5f);
-        const float denom = v == 0.0f ? 0.0f : exp2_entry(half, o.off, o.has);
-        // through the weight product and the quotient; the row sum for the broadcast denominator
-        p = 0.0f;
+        float cen[CH], g[CH], terms[CH];
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            load_row<CH>(cen, x + r * n, n, lane, 0.0f);
+            load_row<CH>(g, gy + r * n, n, lane, 1.0f);
+            GradUnchecked u{o};
+            layer_norm_grad_row<CH>(cen, g, terms, weight, lane, n, count, eps, u);
+            done = __ballot(!u.valid()) == 0ull;
+        }
+        if (!done) {                                    // the row is read again (from cache) rather than kept in registers
+            load_row<CH>(cen, x + r * n, n, lane, 0.0f);
+            load_row<CH>(g, gy + r * n, n, lane, 1.0f);
+            GradChecked k{o, ap};
+            layer_norm_grad_row<CH>(cen, g, terms, weight, lane, n, count, eps, k);
+        }
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const long i = lane + 64L * c;
-            if (i < n) {
-                if (weight) {
-                    const float xn = m.div(cen[c], denom), wi = weight[i];
-                    if (dw_terms) dw_terms[r * n + i] = m.mul_db(xn, wi, g[c]);
-                    g[c] = m.mul_da(xn, wi, g[c]);
-                }
-                p = p + m.div_db(cen[c], denom, g[c]);
-            }
+            if (i < n) { dx[r * n + i] = g[c]; if (weight && dw_terms) dw_terms[r * n + i] = terms[c]; }
         }
-        float d = wave_sum(p);
-        if (v == 0.0f) d = 0.0f;                                   // where(v == 0, 0, exp2(..))
-        d = m.exp2_dx(half, d);
-        d = m.mul_da(lg, 0.5f, d);
-        d = m.log2_dx(v, d);                                       // = d var
-        const float ds2 = m.div_da(s2, count, d);
-        // gradients reaching the centred values: quotient, then the two operands of c (*) c
-        p = 0.0f;
-#pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            if (lane + 64L * c < n) {
-                float dc = m.div_da(cen[c], denom, g[c]);
-                dc = dc + m.mul_da(cen[c], cen[c], ds2);
-                dc = dc + m.mul_db(cen[c], cen[c], ds2);
-                g[c] = dc;
-                p = p + dc;
-            }
-        }
-        const float ds1 = m.div_da(s1, count, -wave_sum(p));       // mu is subtracted: it collects -sum(dc)
-#pragma unroll
-        for (int c = 0; c < CH; ++c) { const long i = lane + 64L * c; if (i < n) dx[r * n + i] = g[c] + ds1; }
     }
 }
 
