@@ -245,8 +245,14 @@ __device__ __forceinline__ uint32_t normalised_fraction(float d)
     return m;
 }
 
+#ifdef PAM_GEMM_WAVES
+#define PAM_GEMM_OCCUPANCY __attribute__((amdgpu_waves_per_eu(PAM_GEMM_WAVES)))
+#else
+#define PAM_GEMM_OCCUPANCY
+#endif
+
 template <int BM, int BN, int TM, int TN, int BK, int MODE, int LKIND, int RKIND>
-__global__ __launch_bounds__((BM / TM) * (BN / TN)) void gemm_kernel(GemmArgs g, float* __restrict__ partial)
+__global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm_kernel(GemmArgs g, float* __restrict__ partial)
 {
     constexpr int TXN = BN / TN, TYN = BM / TM, NT = TXN * TYN, NW = NT / 64;
     constexpr int GM = TM / 4, GN = TN / 4;               // 4-wide groups per micro-tile side
