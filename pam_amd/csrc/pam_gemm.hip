@@ -464,16 +464,43 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     }
 }
 
-// Split-K: Y = ((0 + chunk0) + chunk1) + ... in ascending chunk order.
+// Split-K: Y = ((0 + chunk0) + chunk1) + ... in ascending chunk order.  Loads of several chunks are
+// in flight together; the additions keep their order.
+template <class T>
+__device__ __forceinline__ T splitk_sum(const T* __restrict__ p, int chunks, long stride)
+{
+    T total = T{};
+    int c = 0;
+    for (; c + 8 <= chunks; c += 8) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[(long)(c + u) * stride];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) total += v[u];
+    }
+    for (; c < chunks; ++c) total += p[(long)c * stride];
+    return total;
+}
+
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int chunks, long slab,
                                                            float* __restrict__ y, long y_sb, long y_sr, long y_sc, int M, int N)
 {
     long idx = (long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= slab) return;
-    float total = 0.0f;
-    for (int c = 0; c < chunks; ++c) total += partial[(long)c * slab + idx];
+    const float total = splitk_sum(partial + idx, chunks, slab);
     long b = idx / ((long)M * N), rem = idx % ((long)M * N);
     y[b * y_sb + (rem / N) * y_sr + (rem % N) * y_sc] = total;
+}
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// contiguous output, slab a multiple of four: 128-bit accesses
+__global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const v4f* __restrict__ partial, int chunks, long slab4,
+                                                               v4f* __restrict__ y)
+{
+    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= slab4) return;
+    y[idx] = splitk_sum(partial + idx, chunks, slab4);
 }
 
 int g_cus = 0;
@@ -588,8 +615,14 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     }
     if (p.ksplit > 1) {
         long slab = batch * M * N;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((slab + 255) / 256)), dim3(256), 0, st,
-                           partial, p.ksplit, slab, y, y_sb, y_sr, y_sc, (int)M, (int)N);
+        const bool dense = y_sc == 1 && y_sr == N && (batch == 1 || y_sb == M * N) && slab % 4 == 0 &&
+                           ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(partial)) & 15u) == 0;
+        if (dense && slab / 4 >= 64L * cu_count())         // enough 128-bit lanes to fill the machine
+            hipLaunchKernelGGL(splitk_reduce_vec_kernel, dim3((unsigned)((slab / 4 + 255) / 256)), dim3(256), 0, st,
+                               (const v4f*)partial, p.ksplit, slab / 4, (v4f*)y);
+        else
+            hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((slab + 255) / 256)), dim3(256), 0, st,
+                               partial, p.ksplit, slab, y, y_sb, y_sr, y_sc, (int)M, (int)N);
     }
     return pamhost::check_launch(what);
 }
