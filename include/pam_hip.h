@@ -99,6 +99,12 @@ int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_chunk, int *k_g
 int pam_hip_pam_matmul_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
                            float *y, long y_sr, long y_sc, long m, long n, long k, float offset,
                            void *workspace, size_t workspace_bytes, void *stream);
+/* Y = A (x) B + bias[column]: the product followed by the bias add of pam.linear
+ * (pam/pam_ops.py:107-115) in one pass; the bias is added once to the finished sum (after the chunk
+ * sums when k is split), which is what the separate add computes.  bias NULL = no bias. */
+int pam_hip_pam_linear_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc, const float *bias,
+                           float *y, long y_sr, long y_sc, long m, long n, long k, float offset,
+                           void *workspace, size_t workspace_bytes, void *stream);
 /* batched                                     replaces pam_bmm_fwd (matmul_caller<&pam,true>) */
 int pam_hip_pam_bmm_fwd(PAM_HIP_MAT(a), PAM_HIP_MAT(b), PAM_HIP_OUT(y), long batch, long m, long n, long k,
                         float offset, void *workspace, size_t workspace_bytes, void *stream);

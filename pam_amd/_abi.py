@@ -38,6 +38,7 @@ _SIGNATURES = {
     "pam_hip_gemm_workspace_bytes": ([_l, _l, _l, _l], _z),
     "pam_hip_gemm_plan": ([_l, _l, _l, _l, ctypes.POINTER(_i), ctypes.POINTER(_i)], _i),
     "pam_hip_pam_matmul_fwd": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_pam_linear_fwd": (_MAT2 * 2 + [_p] + _MAT2 + [_l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_bmm_fwd": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_standard_matmul": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_standard_bmm": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
@@ -426,3 +427,23 @@ def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset):
             _call("pam_hip_conv2d_bwd_weight", X.data_ptr(), dY.data_ptr(), W.data_ptr(), dW.data_ptr(), *geo,
                   int(bool(exact)), float(offset), ws.data_ptr(), nbytes, _stream())
     return dW
+
+
+def linear_fwd(X, Wt, bias, offset):
+    """X[m, k] (x) Wt[k, n] + bias[n] in one pass (any strides for X and Wt; bias contiguous or None)."""
+    _check(X, Wt) if bias is None else _check(X, Wt, bias)
+    if X.dim() != 2 or Wt.dim() != 2 or X.shape[1] != Wt.shape[0]:
+        raise ValueError(f"linear_fwd: shapes {tuple(X.shape)} and {tuple(Wt.shape)} do not multiply")
+    m, k = X.shape
+    n = Wt.shape[1]
+    if bias is not None and (bias.numel() != n or not bias.is_contiguous()):
+        raise ValueError("linear_fwd: bias must be contiguous with one value per output column")
+    out = torch.empty((m, n), dtype=torch.float32, device=X.device)
+    if out.numel():
+        with torch.cuda.device(X.device):
+            ws_bytes = load_library().pam_hip_gemm_workspace_bytes(1, m, n, k)
+            ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
+            _call("pam_hip_pam_linear_fwd", X.data_ptr(), X.stride(0), X.stride(1), Wt.data_ptr(), Wt.stride(0), Wt.stride(1),
+                  None if bias is None else bias.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), m, n, k,
+                  float(offset), ws.data_ptr() if ws is not None else None, ws_bytes, _stream())
+    return out

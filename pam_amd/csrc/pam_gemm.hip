@@ -66,6 +66,7 @@ struct GemmArgs {
     ConvGeom cv;
     const float* D; long d_sb, d_sr, d_sc;
     float* Y; long y_sb, y_sr, y_sc;
+    const float* bias;           // one value per output column, added once after the sum, or null
     int M, N, K;
     int ksplit, kchunk;          // kchunk is a multiple of 32; ksplit == 1 means no split
     float off; int has_off;
@@ -445,6 +446,17 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     } else {
         out = g.Y + (long)zb * g.y_sb; o_sr = g.y_sr; o_sc = g.y_sc;
     }
+    if (g.bias && g.ksplit == 1) {           // with split-K the reduction adds it
+#pragma unroll
+        for (int gj = 0; gj < GN; ++gj)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = col0 + gj * (BN / GN) + tx * 4 + j;
+                const float bv = c < g.N ? g.bias[c] : 0.0f;
+#pragma unroll
+                for (int i = 0; i < TM; ++i) acc[i][gj * 4 + j] = acc[i][gj * 4 + j] + bv;
+            }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         int r = row0 + (i / 4) * (BM / GM) + ty * 4 + (i % 4);
@@ -483,12 +495,14 @@ __device__ __forceinline__ T splitk_sum(const T* __restrict__ p, int chunks, lon
 }
 
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int chunks, long slab,
-                                                           float* __restrict__ y, long y_sb, long y_sr, long y_sc, int M, int N)
+                                                           float* __restrict__ y, long y_sb, long y_sr, long y_sc, int M, int N,
+                                                           const float* __restrict__ bias)
 {
     long idx = (long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= slab) return;
-    const float total = splitk_sum(partial + idx, chunks, slab);
+    float total = splitk_sum(partial + idx, chunks, slab);
     long b = idx / ((long)M * N), rem = idx % ((long)M * N);
+    if (bias) total = total + bias[rem % N];
     y[b * y_sb + (rem / N) * y_sr + (rem % N) * y_sc] = total;
 }
 
@@ -496,11 +510,16 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 // contiguous output, slab a multiple of four: 128-bit accesses
 __global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const v4f* __restrict__ partial, int chunks, long slab4,
-                                                               v4f* __restrict__ y)
+                                                               v4f* __restrict__ y, const float* __restrict__ bias, int N)
 {
     long idx = (long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= slab4) return;
-    y[idx] = splitk_sum(partial + idx, chunks, slab4);
+    v4f total = splitk_sum(partial + idx, chunks, slab4);
+    if (bias) {                                   // N is a multiple of four here: the four lanes share a row
+        const int c = (int)((idx * 4) % N);
+        total.x = total.x + bias[c]; total.y = total.y + bias[c + 1]; total.z = total.z + bias[c + 2]; total.w = total.w + bias[c + 3];
+    }
+    y[idx] = total;
 }
 
 int g_cus = 0;
@@ -579,7 +598,8 @@ void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& 
 int gemm(const char* what, int mode, long batch, long M, long N, long K,
          const float* l, long l_sb, long l_sr, long l_sc, const float* r, long r_sb, long r_sr, long r_sc,
          const float* d, long d_sb, long d_sr, long d_sc, float* y, long y_sb, long y_sr, long y_sc,
-         float offset, void* workspace, size_t workspace_bytes, void* stream, const ConvGeom* conv = nullptr)
+         float offset, void* workspace, size_t workspace_bytes, void* stream, const ConvGeom* conv = nullptr,
+         const float* bias = nullptr)
 {
     if (batch < 0 || M < 0 || N < 0 || K < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: negative size", what);
     if (batch == 0 || M == 0 || N == 0) return PAM_HIP_OK;
@@ -599,6 +619,7 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     g.R = Operand{r, r_sb, r_sc, r_sr};            // R's "row" index is the output column
     g.D = d; g.d_sb = d_sb; g.d_sr = d_sr; g.d_sc = d_sc;
     g.Y = y; g.y_sb = y_sb; g.y_sr = y_sr; g.y_sc = y_sc;
+    g.bias = bias;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.ksplit = p.ksplit; g.kchunk = p.kchunk;
     g.off = offset; g.has_off = (mode != MODE_STD && offset != 1.0f) ? 1 : 0;
@@ -616,14 +637,14 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     }
     if (p.ksplit > 1) {
         long slab = batch * M * N;
-        const bool dense = y_sc == 1 && y_sr == N && (batch == 1 || y_sb == M * N) && slab % 4 == 0 &&
+        const bool dense = y_sc == 1 && y_sr == N && (batch == 1 || y_sb == M * N) && slab % 4 == 0 && (!bias || N % 4 == 0) &&
                            ((reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(partial)) & 15u) == 0;
         if (dense && slab / 4 >= 64L * cu_count())         // enough 128-bit lanes to fill the machine
             hipLaunchKernelGGL(splitk_reduce_vec_kernel, dim3((unsigned)((slab / 4 + 255) / 256)), dim3(256), 0, st,
-                               (const v4f*)partial, p.ksplit, slab / 4, (v4f*)y);
+                               (const v4f*)partial, p.ksplit, slab / 4, (v4f*)y, bias, (int)N);
         else
             hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((slab + 255) / 256)), dim3(256), 0, st,
-                               partial, p.ksplit, slab, y, y_sb, y_sr, y_sc, (int)M, (int)N);
+                               partial, p.ksplit, slab, y, y_sb, y_sr, y_sc, (int)M, (int)N, bias);
     }
     return pamhost::check_launch(what);
 }
@@ -719,6 +740,14 @@ int pam_hip_pam_matmul_fwd(const float* a, long a_sr, long a_sc, const float* b,
 {
     return gemm("pam_matmul_fwd", MODE_PAM, 1, m, n, k, a, 0, a_sr, a_sc, b, 0, b_sr, b_sc, nullptr, 0, 0, 0,
                 y, 0, y_sr, y_sc, offset, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_pam_linear_fwd(const float* a, long a_sr, long a_sc, const float* b, long b_sr, long b_sc, const float* bias,
+                           float* y, long y_sr, long y_sc, long m, long n, long k, float offset,
+                           void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemm("pam_linear_fwd", MODE_PAM, 1, m, n, k, a, 0, a_sr, a_sc, b, 0, b_sr, b_sc, nullptr, 0, 0, 0,
+                y, 0, y_sr, y_sc, offset, workspace, workspace_bytes, stream, nullptr, bias);
 }
 
 int pam_hip_pam_bmm_fwd(PAM_HIP_MAT(a), PAM_HIP_MAT(b), PAM_HIP_OUT(y), long batch, long m, long n, long k,

@@ -201,3 +201,42 @@ class conv2d_autograd(torch.autograd.Function):
 
 def conv2d(X, W, stride, padding, offset=None, approx_bwd=False):
     return conv2d_autograd.apply(X, W, tuple(stride), tuple(padding), offset, approx_bwd)
+
+
+# ---------------------------------------------------------------- linear with the bias added in the product's epilogue
+
+class linear_autograd(torch.autograd.Function):
+    """X W^T + bias in one kernel; the gradients are those of the product
+    (pam/cuda_bindings.py:132-166) and, for the bias, the sum of the upstream gradient over the rows."""
+
+    @staticmethod
+    def forward(ctx, X, W, bias, offset, approx_bwd):
+        ctx.offset = _offset_value(offset)
+        ctx.approx_bwd = approx_bwd
+        X2, _ = cuda_bindings.check_row_major(X, 2)
+        Wt, _ = cuda_bindings.check_row_major(W.t(), 2)
+        ctx.save_for_backward(X2, Wt)
+        return _abi.linear_fwd(X2, Wt, bias.contiguous(), ctx.offset)
+
+    @staticmethod
+    def backward(ctx, dY):
+        A, B = ctx.saved_tensors                      # A = X, B = W^T as the product saw them
+        k, off = cuda_bindings.cuda_kernels, ctx.offset
+        approx_a, approx_b = _both(ctx.approx_bwd)
+        crm = cuda_bindings.check_row_major
+        dY2, dY_rm = crm(dY, 2)
+        At, At_rm = crm(A.mT, 2)
+        Bt, Bt_rm = crm(B.mT, 2)
+        dX = dW = db = None
+        if ctx.needs_input_grad[0]:
+            dX = k.pam_matmul_fwd(dY2, Bt, dY_rm, Bt_rm, off) if approx_a else k.pam_matmul_bwd(dY2, Bt, A, dY_rm, Bt_rm, True, off)
+        if ctx.needs_input_grad[1]:
+            dB = k.pam_matmul_fwd(At, dY2, At_rm, dY_rm, off) if approx_b else k.pam_matmul_bwd(At, dY2, B, At_rm, dY_rm, False, off)
+            dW = dB.t()
+        if ctx.needs_input_grad[2]:
+            db = dY2.sum(0)
+        return dX, dW, db, None, None
+
+
+def linear_with_bias(X2d, W, bias, offset=None, approx_bwd=False):
+    return linear_autograd.apply(X2d, W, bias, offset, approx_bwd)

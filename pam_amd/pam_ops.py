@@ -11,9 +11,12 @@ import math
 import torch
 
 from . import cuda_bindings
+from . import fused
 from . import utils
 
 __all__ = ["mul", "div", "exp", "exp2", "log", "log2", "pow", "matmul", "bmm", "linear", "Linear"]
+
+fused_bias = True        # False: linear() adds the bias with a separate torch add, as the reference does
 
 
 def _require_kernel(t, use_kernel):
@@ -98,7 +101,13 @@ def linear(X, W, bias=None, *, offset=None, approx_bwd=False, use_kernel=True):
     """X W^T + bias with PAM products; leading dims are flattened like torch.nn.Linear
     (pam/pam_ops.py:107-115).  W.T is passed as a view: the kernel reads W in place."""
     lead = X.shape[:-1]
-    out = matmul(X.reshape(-1, X.shape[-1]), W.T, offset=offset, approx_bwd=approx_bwd, use_kernel=use_kernel)
+    rows = X.reshape(-1, X.shape[-1])
+    if (fused_bias and bias is not None and use_kernel and rows.is_cuda and rows.numel() and bias.dim() == 1
+            and all(t.dtype == torch.float32 for t in (rows, W, bias))):
+        # the bias is added to the finished sums inside the product kernel: the same add, one pass less
+        out = fused.linear_with_bias(rows, W, bias, offset, approx_bwd)
+        return out.reshape(*lead, out.shape[-1])
+    out = matmul(rows, W.T, offset=offset, approx_bwd=approx_bwd, use_kernel=use_kernel)
     out = out.reshape(*lead, out.shape[-1])
     return out if bias is None else out + bias
 

@@ -414,3 +414,37 @@ def test_reference_vectors_on_device(K):
     g = np.load(GOLDEN / "matmul_small.npz")
     assert_same_bits(host(C), f32(g["p20_c"]).reshape(5, 3), "reference 5x4 @ 4x3 forward")
     assert np.allclose(host(A.grad), f32(g["p20_da_approx"]).reshape(5, 4)) and np.allclose(host(B.grad), f32(g["p20_db_approx"]).reshape(4, 3))
+
+
+@pytest.mark.gpu
+def test_linear_with_bias_in_the_epilogue(oracle):
+    """pam.linear with a bias: added inside the product kernel (after the chunk sums when k is split),
+    bit-identical to the product followed by a separate add; gradients as without the fusion."""
+    import pam_amd
+    from pam_amd import pam_ops, _abi
+    rng = np.random.RandomState(11)
+    for (m, k, n) in [(197, 192, 768), (50, 1000, 24), (7, 5, 3), (3000, 4096, 64)]:
+        X = rng.standard_normal((m, k)).astype(np.float32); W = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+        b = rng.standard_normal(n).astype(np.float32); dY = rng.standard_normal((m, n)).astype(np.float32)
+        want = (ogemm(oracle, X, W.T) + b).astype(np.float32)
+        res = {}
+        for fused_on in (True, False):
+            pam_ops.fused_bias = fused_on
+            try:
+                x = torch.from_numpy(X).cuda().requires_grad_(); w = torch.from_numpy(W).cuda().requires_grad_()
+                bb = torch.from_numpy(b).cuda().requires_grad_()
+                y = pam_amd.linear(x, w, bb, approx_bwd=True, offset=None)
+                y.backward(torch.from_numpy(dY).cuda())
+                res[fused_on] = [t.detach().cpu().numpy() for t in (y, x.grad, w.grad, bb.grad)]
+            finally:
+                pam_ops.fused_bias = True
+        assert_same_bits(res[True][0], want, f"linear+bias {m}x{k}x{n}")
+        for a, c, name in zip(res[True], res[False], ("y", "dX", "dW", "db")):
+            assert_same_bits(a, c, f"{name} fused vs separate add, {m}x{k}x{n}")
+    # leading dimensions and the module
+    lin = pam_amd.Linear(192, 96, approx_bwd=True).cuda()
+    x3 = torch.randn(4, 197, 192, device="cuda")
+    pam_ops.fused_bias = False
+    ref = lin(x3)
+    pam_ops.fused_bias = True
+    assert torch.equal(lin(x3), ref) and lin(x3).shape == (4, 197, 96)
