@@ -32,10 +32,13 @@
  *   pa_log2 / pa_exp2 / pa_exp / pa_log  native goldens
  *   chain flavour .................... native goldens (bit-for-bit outside the
  *                                      log2f glitch band)
- *   pad_bwd, pa_exp_bwd, pa_log_bwd .. PARITY UNPINNED beyond the closed forms of
- *                                      pam/cuda_kernels.cu:85-136,375-393,470-486:
- *                                      the reference has no CPU implementation and
- *                                      no test of them.
+ *   pad_bwd, pa_exp_bwd, pa_log_bwd .. closed forms of pam/cuda_kernels.cu:85-136,
+ *                                      375-393,470-486 (the reference has no CPU
+ *                                      implementation, test or vector of them), pinned
+ *                                      as the slope of the pinned forward functions by
+ *                                      finite differences inside one affine piece
+ *                                      (pad_bwd up to the reference's sign convention
+ *                                      for negative divisors, which the test states).
  *   row-wise compositions ............ equal, bit for bit, to the same chain built from
  *                                      the pinned primitives above whenever the row sums
  *                                      are exact (short-mantissa rows), and to it within

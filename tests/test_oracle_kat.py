@@ -157,6 +157,38 @@ def test_pam_bwd_is_slope_of_forward(oracle):
     assert inside.sum() > 2000 and (slope[inside] == (np.sign(b) * got)[inside]).all()
 
 
+def test_exp_log_bwd_are_slopes_of_forward(oracle):
+    """pa_exp_bwd / pa_log_bwd (closed forms of pam/cuda_kernels.cu:375-393, 470-486, for which the
+    reference holds no CPU implementation and no test) against the derivative of the pinned forward
+    functions: both are piecewise affine with power-of-two slopes, so a finite difference inside one
+    affine piece gives the slope up to the rounding of the forward values."""
+    rng = np.random.RandomState(6)
+    n = 6000
+    for base in (math.e, 2.0, 10.0):
+        for off in (None, 1.0552):
+            # exp: x with short mantissas; keep the points whose neighbours share the affine piece
+            x = ((1 + rng.randint(1, 2 ** 10 - 1, n) / 2.0 ** 10) * 2.0 ** rng.randint(-3, 3, n) * rng.choice([-1, 1], n)).astype(np.float32)
+            h = (np.abs(x) * 2.0 ** -10).astype(np.float32)
+            f0, f1, f2 = (oracle.pa_exp(v, base, off).astype(np.float64) for v in (x - h, x, x + h))
+            got = oracle.pa_exp_bwd(x, np.ones_like(x), base, off).astype(np.float64)
+            left, right = (f1 - f0) / h, (f2 - f1) / h
+            same_piece = np.abs(left / right - 1) < 2.0 ** -9               # no kink between x - h and x + h
+            assert same_piece.sum() > n // 2
+            assert (np.abs(right[same_piece] / got[same_piece] - 1) < 2.0 ** -7).all(), (base, off)
+            # log: positive x
+            y = np.abs(x)
+            hy = (y * 2.0 ** -10).astype(np.float32)
+            g0, g1, g2 = (oracle.pa_log(v, base, off).astype(np.float64) for v in (y - hy, y, y + hy))
+            got = oracle.pa_log_bwd(y, np.ones_like(y), base, off).astype(np.float64)
+            left, right = (g1 - g0) / hy, (g2 - g1) / hy
+            same_piece = (np.abs(left / right - 1) < 2.0 ** -9) & (g1 != g0) & (np.abs(y - 1) > 2.0 ** -6)   # log2 near 0 runs through many pieces
+            assert same_piece.sum() > n // 2
+            assert (np.abs(right[same_piece] / got[same_piece] - 1) < 2.0 ** -6).all(), (base, off)
+    # upstream gradient scales linearly
+    x = np.array([0.7, -1.3, 2.5], np.float32); d = np.array([2.0, -4.0, 0.5], np.float32)
+    assert_same_bits(oracle.pa_exp_bwd(x, d), (oracle.pa_exp_bwd(x, np.ones(3, np.float32)) * d).astype(np.float32), "linear in dy")
+
+
 def test_gemm_power_of_two_equals_matmul(oracle):
     # construction of pam/test_pam.py:198-216: right operand all powers of two => PAM bmm == bmm
     rng = np.random.RandomState(4)
