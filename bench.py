@@ -177,6 +177,10 @@ def main():
         pr = torch.softmax(torch.randn(Bh, Tk, Tk, generator=g), -1).to(dev)
         exact["bmm_QKt_192x197x197x64"] = (2, Bh * Tk * Tk * Dh, lambda: K.pam_bmm_fwd(q, kk.transpose(1, 2), True, False, 1.0))
         exact["bmm_PV_192x197x64x197"] = (2, Bh * Tk * Tk * Dh, lambda: K.pam_bmm_fwd(pr, v, True, True, 1.0))
+        # operands with zeros: ReLU output as the left operand (the second layer of a ReLU feed-forward block)
+        X2r = torch.relu(X2)
+        exact["fwd_12608x192x768_relu_input"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2r, W2.T, True, False, 1.0))
+        exact["dW_768x192x12608_relu_input"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2r.T, dY2, False, True, 1.0))
         for name, (ops, macs, fn) in exact.items():
             ms = event_time_ms(fn, 10, torch)
             other[name] = {"ms": round(ms, 4), "gmacs": round(macs / ms / 1e6, 1), "valu_frac": round(ops * macs / (ms * 1e-3) / lane_peak, 4)}

@@ -26,8 +26,9 @@
 //  * While staging, every element's exponent is folded into a running min/max.  If all of a
 //    k-tile's L and R values are normal numbers with magnitude in [2^-63, 2^64), no product
 //    in the tile can leave the normal range and the two-instruction loop is exact;
-//    a k-tile that only adds zeros to that (ReLU activations, padding) takes a loop with one
-//    extra select per product; anything else (subnormals, inf, NaN, extreme exponents) takes a
+//    a k-tile that only adds zeros to that in one operand (ReLU activations, padding) keeps two
+//    instructions per product: the zero becomes a stand-in value and the accumulating fma
+//    multiplies the product by 0 or 1; zeros in both operands cost one select per product; anything else (subnormals, inf, NaN, extreme exponents) takes a
 //    guarded loop that evaluates the full definition per product on operands decomposed once
 //    per k-step.  The choice is uniform per work-group and k-tile.
 //  * Rows beyond M / N are clamped to the last valid row when loading (their results are
@@ -105,11 +106,19 @@ struct Stager {
         emin = min(emin, e); emax = max(emax, e);
         return u;
     }
-    // 2: some staged value lies outside [2^-63, 2^64) or is not a normal number or zero;
-    // 1: all non-zero values are inside, but there are zeros; 0: the plain loop is exact
-    __device__ __forceinline__ uint32_t verdict() const
-    { return (bad || emin < 64u || emax > 190u) ? 2u : zero ? 1u : 0u; }
+    // some staged value lies outside [2^-63, 2^64) or is not a normal number or zero
+    __device__ __forceinline__ bool out_of_range() const { return bad || emin < 64u || emax > 190u; }
 };
+
+// Verdict of a k-tile: bit 0 / bit 1 = the left / right operand holds zeros (all else in range),
+// kGuarded = some value needs the full definition.  Verdicts of wavefronts combine by OR.
+constexpr uint32_t kZerosL = 1u, kZerosR = 2u, kGuarded = 4u;
+
+// Stand-ins that keep the integer sum a finite number when one operand is zero: 2^-64 on the
+// left, 2^64 (less the bias) on the right, just outside the range [2^-63, 2^64) that the other
+// values of such a k-tile lie in.  The product is then multiplied by 0.
+constexpr uint32_t kStandInL = 63u << 23;
+constexpr uint32_t kStandInR = 64u << 23;
 
 // One operand's tile: ROWS x BK values from global memory into registers, then into LDS.
 template <int ROWS, int NT, int KIND, int BK>
@@ -219,6 +228,15 @@ struct TileLoader {
     }
 };
 
+// Per-lane choice by a wavefront mask (as __ballot returns it): one v_cndmask, kept opaque so that the
+// 0 / 1 factor of the zero-skipping loops stays a factor and is not turned back into a select per product.
+__device__ __forceinline__ uint32_t pick(uint64_t mask, uint32_t if_clear, uint32_t if_set)
+{
+    uint32_t r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(if_clear), "v"(if_set), "s"(mask));
+    return r;
+}
+
 // Exact-backward product from the normalised mantissa fraction of the forward operand
 // whose gradient is wanted, the other forward operand b (offset already applied) and the
 // upstream gradient (pam/cuda_kernels.cu:48-57, pam/native.py:74-77), all classes.
@@ -309,9 +327,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         ll.store(lds_l[buf], tid, sl);
         rl.store(lds_r[buf], tid, sr);
         if (MODE != MODE_STD) {
-            uint32_t v = max(sl.verdict(), sr.verdict());
-            uint32_t worst = __ballot(v == 2u) != 0ull ? 2u : __ballot(v == 1u) != 0ull ? 1u : 0u;
-            if (lane == 0) lds_flag[buf][wave] = worst;
+            const uint32_t found = (__ballot(sl.out_of_range() || sr.out_of_range()) != 0ull ? kGuarded : 0u)
+                                 | (__ballot(sl.zero) != 0ull ? kZerosL : 0u) | (__ballot(sr.zero) != 0ull ? kZerosR : 0u);
+            if (lane == 0) lds_flag[buf][wave] = found;
         }
     };
 
@@ -331,11 +349,11 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid, g.cv);
         rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid, g.cv);
         const int kcount = min(BK, kend - k0);
-        uint32_t verdict = 0;                     // 0 plain loop, 1 zeros present, 2 guarded
+        uint32_t verdict = 0;                     // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
         if (MODE != MODE_STD) {
             uint32_t f = 0;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) f = max(f, lds_flag[cur][w]);
+            for (int w = 0; w < NW; ++w) f |= lds_flag[cur][w];
             verdict = __builtin_amdgcn_readfirstlane(f);
         }
         const uint32_t* sl = lds_l[cur] + ty * 4;
@@ -380,6 +398,40 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[i][j] += u2f((za[i] | zb[j]) ? 0u : a[i] + b[j]);
+        };
+        // zeros in one operand only: its zeros become a stand-in that keeps the integer sum finite, and
+        // the product is multiplied by 0 or 1 in the accumulating fma (x * 1 + acc rounds like acc + x;
+        // x * 0 + acc leaves acc, which is never -0) -- two instructions per product like the plain loop,
+        // plus three per value of the operand with zeros
+        auto zeros_left_step = [&](int kk) {
+            uint32_t a[TM], b[TN];
+            fragment(kk, a, b);
+            float keep[TM];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const uint64_t nonzero = __ballot(a[i] != kZeroL);
+                keep[i] = u2f(pick(nonzero, 0u, 0x3f800000u));
+                a[i] = max(a[i], kStandInL);          // every other value is larger, as an unsigned number
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[i], acc[i][j]);
+        };
+        auto zeros_right_step = [&](int kk) {
+            uint32_t a[TM], b[TN];
+            fragment(kk, a, b);
+            float keep[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const uint64_t nonzero = __ballot(b[j] != kZeroR);
+                keep[j] = u2f(pick(nonzero, 0u, 0x3f800000u));
+                b[j] = pick(nonzero, kStandInR, b[j]);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[j], acc[i][j]);
         };
         auto guarded_step = [&](int kk) {
             uint32_t a[TM], b[TN];
@@ -427,7 +479,13 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 #pragma unroll 1
                 for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
             }
-        } else if (verdict == 1 && MODE == MODE_PAM) {
+        } else if (verdict == kZerosL && MODE == MODE_PAM) {
+#pragma unroll 2
+            for (int kk = 0; kk < kcount; ++kk) zeros_left_step(kk);
+        } else if (verdict == kZerosR && MODE == MODE_PAM) {
+#pragma unroll 2
+            for (int kk = 0; kk < kcount; ++kk) zeros_right_step(kk);
+        } else if (verdict == (kZerosL | kZerosR) && MODE == MODE_PAM) {
 #pragma unroll 2
             for (int kk = 0; kk < kcount; ++kk) zeros_step(kk);
         } else {

@@ -219,6 +219,34 @@ def test_matmul_zeros_and_specials(K, oracle, zeros, specials):
     assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), ogemm(oracle, A, B, offset=1.0552), "offset")
 
 
+@pytest.mark.parametrize("side", ["left", "right", "mixed"])
+def test_matmul_zeros_in_one_operand(K, oracle, side):
+    """k-tiles whose zeros sit in one operand only take their own loop (a stand-in for the zero and a
+    0 / 1 factor in the accumulating fma): signed zeros, values at both ends of the range that this
+    loop accepts, and in the mixed case k-tiles of all four kinds (none, left, right, both) in one product."""
+    rng = np.random.RandomState(21)
+    A, B = _rand((140, 192), 31), _rand((192, 130), 32)
+    edge = np.array([2.0 ** -63, -(2.0 ** -63), np.nextafter(np.float32(2.0 ** 64), np.float32(0)), -1.5 * 2.0 ** 63], np.float32)
+    A.reshape(-1)[rng.choice(A.size, 64, replace=False)] = np.resize(edge, 64)
+    B.reshape(-1)[rng.choice(B.size, 64, replace=False)] = np.resize(edge, 64)
+    za, zb = rng.rand(*A.shape) < 0.4, rng.rand(*B.shape) < 0.4
+    if side == "left":
+        zb[:] = False
+    elif side == "right":
+        za[:] = False
+    else:                           # k in [0,32) none, [32,64) left, [64,96) right, [96,128) both, then left / right again
+        za[:, :32] = False; zb[:32] = False; zb[32:64] = False; za[:, 64:96] = False; zb[128:160] = False; za[:, 160:] = False
+    A[za] = np.where(rng.rand(int(za.sum())) < 0.5, 0.0, -0.0)
+    B[zb] = np.where(rng.rand(int(zb.sum())) < 0.5, 0.0, -0.0)
+    for la, ta in _layouts(A).items():
+        for lb, tb in _layouts(B).items():
+            assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), ogemm(oracle, A, B), f"{side}: {la} x {lb}")
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), ogemm(oracle, A, B, offset=1.0552), "offset")
+    # an all-zero row / column keeps its +0 sums
+    A[3] = 0.0; B[:, 5] = -0.0
+    assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)), ogemm(oracle, A, B), "zero row and column")
+
+
 @pytest.mark.parametrize("delta_l", [True, False])
 @pytest.mark.parametrize("zeros,specials", [(0.0, False), (0.3, True)])
 def test_matmul_exact_backward(K, oracle, delta_l, zeros, specials):
