@@ -174,7 +174,8 @@ int pam_hip_layer_norm_bwd(const float *x, const float *weight, const float *dy,
  * output size (in + 2 pad - k) / stride + 1.  Sums run over k = (c, i, j) in ascending order in
  * the chunks pam_hip_gemm_plan(batch, co, ho*wo, c*kh*kw) reports. */
 size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
-                                      long stride_h, long stride_w, long pad_h, long pad_w, int weight_gradient, float offset);
+                                      long stride_h, long stride_w, long pad_h, long pad_w, int which, float offset);
+/* which: 0 forward, 1 weight gradient, 2 input gradient */
 /* y[batch][co][ho][wo] = sum_k x_patch (*) (w (*) offset)           replaces pam.conv2d's forward */
 int pam_hip_conv2d_fwd(const float *x, const float *w, float *y, long batch, long c, long h, long wd, long co, long kh, long kw,
                        long stride_h, long stride_w, long pad_h, long pad_w, float offset,
@@ -186,6 +187,19 @@ int pam_hip_conv2d_fwd(const float *x, const float *w, float *y, long batch, lon
 int pam_hip_conv2d_bwd_weight(const float *x, const float *dy, const float *w, float *dw, long batch, long c, long h, long wd,
                               long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
                               int exact, float offset, void *workspace, size_t workspace_bytes, void *stream);
+
+/* dx[batch][c][h][w] for stride 1 (any other stride is an argument error: the caller keeps the
+ * unfolded path) and pad <= k - 1: the gradient of the input is the convolution of dy, padded by
+ * k - 1 - pad, with the weights flipped and their channel indices exchanged, so it runs on the same
+ * kernel with dy's patches read in place instead of through the [c*kh*kw, ho*wo] gradient of the
+ * unfolded matrix and its overlap-add.  exact == 0: sum_k (w (*) offset) (*) dy_patch
+ * (pam/cuda_bindings.py:157-158); exact != 0: sum_k pam_bwd(x, w, dy_patch) (:158-159), x required
+ * (one x per output element: every patch entry that an input pixel fills is that pixel).
+ * Sums run over k = (co, i, j) ascending in the chunks pam_hip_gemm_plan(batch, c, h*w, co*kh*kw)
+ * reports; the reference's order is that of its matrix kernel followed by torch's fold. */
+int pam_hip_conv2d_bwd_input(const float *dy, const float *w, const float *x, float *dx, long batch, long c, long h, long wd,
+                             long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                             int exact, float offset, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- optimizer step ---------------------------------------------------------------------- */
 /* One Adam update of n parameters in place, every product, the quotient and the square root

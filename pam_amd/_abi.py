@@ -47,6 +47,7 @@ _SIGNATURES = {
     "pam_hip_conv2d_workspace_bytes": ([_l] * 11 + [_i, _f], _z),
     "pam_hip_conv2d_fwd": ([_p, _p, _p] + [_l] * 11 + [_f, _p, _z, _p], _i),
     "pam_hip_conv2d_bwd_weight": ([_p, _p, _p, _p] + [_l] * 11 + [_i, _f, _p, _z, _p], _i),
+    "pam_hip_conv2d_bwd_input": ([_p, _p, _p, _p] + [_l] * 11 + [_i, _f, _p, _z, _p], _i),
     "pam_hip_adam_step": ([_p, _p, _p, _p, _z, _f, _f, _f, _f, _f, _f, _i, _f, _f, _p], _i),
     "pam_hip_rowop_workspace_bytes": ([], _z),
     "pam_hip_softmax_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
@@ -427,6 +428,24 @@ def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset):
             _call("pam_hip_conv2d_bwd_weight", X.data_ptr(), dY.data_ptr(), W.data_ptr(), dW.data_ptr(), *geo,
                   int(bool(exact)), float(offset), ws.data_ptr(), nbytes, _stream())
     return dW
+
+
+def conv2d_bwd_input(dY, W, X, padding, exact, offset):
+    """dX[batch, c, h, w] of a stride-1 convolution with dY's patches read in place; X gives the
+    shape and, for the exact variant, the values."""
+    _check(dY, W, X)
+    dY, W, X = dY.contiguous(), W.contiguous(), X.contiguous()
+    geo = _conv_geometry(X, W, (1, 1), padding)
+    dX = torch.empty_like(X)
+    if dX.numel():
+        with torch.cuda.device(X.device):
+            nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 2, float(offset))
+            if nbytes == 0:
+                raise ValueError("conv2d_bwd_input: needs stride 1 and padding <= kernel - 1")
+            ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=X.device)
+            _call("pam_hip_conv2d_bwd_input", dY.data_ptr(), W.data_ptr(), X.data_ptr(), dX.data_ptr(), *geo,
+                  int(bool(exact)), float(offset), ws.data_ptr(), nbytes, _stream())
+    return dX
 
 
 def linear_fwd(X, Wt, bias, offset):

@@ -165,7 +165,7 @@ def conv2d(X, W, bias=None, stride=1, padding=0, dilation=1, *, offset=None, app
     batch = X.shape[0]
     c_out, _, kh, kw = W.shape
     padding, stride, (h_out, w_out) = _conv_geometry(X.shape[2:], (kh, kw), stride, padding)
-    if implicit_conv and use_kernel and fused.conv_in_place(X, W, dilation, approx_bwd):
+    if implicit_conv and use_kernel and fused.conv_in_place(X, W, dilation, approx_bwd, stride, padding):
         out = fused.conv2d(X, W, stride, padding, offset, approx_bwd)        # patches read in place
         return out if bias is None else out + bias.view((1, -1, 1, 1))
     patches = torch.nn.functional.unfold(X, (kh, kw), padding=padding, stride=stride, dilation=dilation)

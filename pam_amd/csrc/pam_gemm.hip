@@ -103,6 +103,9 @@ struct Stager {
             emin = min(emin, e); emax = max(emax, e);
             return z ? (IS_R ? kZeroR : kZeroL) : (IS_R ? u - kBias : u);
         }
+        // slope side of a backward mode: a zero needs no care, (0 + fraction) & ~mantissa is 0 and the
+        // fma then adds delta * 0 (delta is finite in the plain loop), which is what the definition gives
+        if ((u & ~kSign) == 0) return u;
         emin = min(emin, e); emax = max(emax, e);
         return u;
     }
@@ -639,7 +642,7 @@ void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, 
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
-    if constexpr (MODE == MODE_PAM || MODE == MODE_BWD_DL) {           // image patches as the right operand
+    if constexpr (MODE != MODE_STD) {                                  // image patches as the right operand
         PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_RVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_ANY, LOAD_CONV)
     }
 #undef PAM_GEMM_CASE
@@ -729,6 +732,18 @@ __global__ __launch_bounds__(256) void scale_kernel(const float* __restrict__ in
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) out[i] = pam_mul(in[i], off);
 }
 
+// wf[c][co][i][j] = w[co][c][kh-1-i][kw-1-j] (*) off: the weights of the convolution over the
+// upstream gradient that yields the gradient of the input (stride 1)
+__global__ __launch_bounds__(256) void flip_weights_kernel(const float* __restrict__ w, float* __restrict__ wf, int c, int co, int kh, int kw,
+                                                          float off, int has_off)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= c * co * kh * kw) return;
+    const int j = idx % kw, i = (idx / kw) % kh, o = (idx / (kw * kh)) % co, ci = idx / (kw * kh * co);
+    const float v = w[(((long)o * c + ci) * kh + (kh - 1 - i)) * kw + (kw - 1 - j)];
+    wf[idx] = has_off ? pam_mul(v, off) : v;
+}
+
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
 
 int conv_shape(const char* what, ConvShape& s)
@@ -768,6 +783,30 @@ int conv_prepare(const char* what, const ConvShape& s, const ConvSpace& sp, void
                        (int)s.kh, (int)s.kw, (int)s.h, (int)s.w, (int)s.wo, (int)s.sh, (int)s.sw, (int)s.ph, (int)s.pw);
     cv = ConvGeom{ktab, ltab, (int)s.h, (int)s.w, transposed ? 1 : 0};
     return PAM_HIP_OK;
+}
+
+// The gradient of the input of a stride-1 convolution is itself a convolution: of the upstream
+// gradient [co, ho, wo], padded by (k - 1 - pad), with the weights flipped and their two channel
+// indices exchanged.  `t` is that convolution's geometry (its "image" is the upstream gradient).
+int input_gradient_shape(const char* what, const ConvShape& s, ConvShape& t)
+{
+    if (s.sh != 1 || s.sw != 1) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: the input gradient in place needs stride 1", what);
+    if (s.ph > s.kh - 1 || s.pw > s.kw - 1) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: padding larger than kernel - 1", what);
+    t = ConvShape{s.batch, s.co, s.ho, s.wo, s.c, s.kh, s.kw, 1, 1, s.kh - 1 - s.ph, s.kw - 1 - s.pw, 0, 0};
+    int rc = conv_shape(what, t);
+    if (rc != PAM_HIP_OK) return rc;
+    if (t.ho != s.h || t.wo != s.w) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: geometry does not invert", what);
+    return PAM_HIP_OK;
+}
+
+// workspace: [k table][l table][flipped weights][split-k partial tiles]
+ConvSpace input_gradient_space(const ConvShape& t)
+{
+    ConvSpace w;
+    w.tables = align256((size_t)(t.K() + t.L()) * sizeof(int2));
+    w.scaled = align256((size_t)t.co * t.K() * sizeof(float));
+    w.total = w.tables + w.scaled + pam_hip_gemm_workspace_bytes(t.batch, t.co, t.L(), t.K());
+    return w;
 }
 
 }  // namespace
@@ -850,11 +889,47 @@ int pam_hip_pam_bmm_bwd(PAM_HIP_MAT(l), PAM_HIP_MAT(r), PAM_HIP_MAT(mo), PAM_HIP
 }
 
 size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
-                                      long stride_h, long stride_w, long pad_h, long pad_w, int weight_gradient, float offset)
+                                      long stride_h, long stride_w, long pad_h, long pad_w, int which, float offset)
 {
     ConvShape s{batch, c, h, w, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
     if (conv_shape("conv2d_workspace_bytes", s) != PAM_HIP_OK || batch == 0) return 0;
-    return conv_space(s, weight_gradient != 0, offset != 1.0f).total;
+    if (which == 2) {
+        ConvShape t;
+        if (input_gradient_shape("conv2d_workspace_bytes", s, t) != PAM_HIP_OK) return 0;
+        return input_gradient_space(t).total;
+    }
+    return conv_space(s, which != 0, offset != 1.0f).total;
+}
+
+int pam_hip_conv2d_bwd_input(const float* dy, const float* w, const float* x, float* dx, long batch, long c, long h, long wd,
+                             long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                             int exact, float offset, void* workspace, size_t workspace_bytes, void* stream)
+{
+    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    int rc = conv_shape("conv2d_bwd_input", s);
+    if (rc != PAM_HIP_OK) return rc;
+    ConvShape t;
+    rc = input_gradient_shape("conv2d_bwd_input", s, t);
+    if (rc != PAM_HIP_OK) return rc;
+    if (batch == 0) return PAM_HIP_OK;
+    if (!dy || !w || !dx || (exact && !x)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_bwd_input: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    ConvSpace sp = input_gradient_space(t);
+    ConvGeom cv;
+    rc = conv_prepare("conv2d_bwd_input", t, sp, workspace, workspace_bytes, st, cv, false);
+    if (rc != PAM_HIP_OK) return rc;
+    float* wf = (float*)((char*)workspace + sp.tables);
+    const long n = c * co * kh * kw;
+    // approximate: the offset goes into the flipped weights; exact: the product kernel applies it to its slope operand
+    hipLaunchKernelGGL(flip_weights_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w, wf, (int)c, (int)co, (int)kh, (int)kw,
+                       offset, (!exact && offset != 1.0f) ? 1 : 0);
+    const long K = t.K(), L = t.L();                  // K = co kh kw, L = h w
+    void* rest = (char*)workspace + sp.tables + sp.scaled; size_t rest_bytes = workspace_bytes - sp.tables - sp.scaled;
+    if (exact)        // dX[c, l] = sum_k pam_bwd(x[c, l], wf[c, k], dY patch[k, l]): x is the same for every term of an output
+        return gemm("conv2d_bwd_input", MODE_BWD_DR, batch, c, L, K, wf, 0, K, 1, dy, co * s.ho * s.wo, 0, 0, x, c * L, L, 1,
+                    dx, c * L, L, 1, offset, rest, rest_bytes, stream, &cv);
+    return gemm("conv2d_bwd_input", MODE_PAM, batch, c, L, K, wf, 0, K, 1, dy, co * s.ho * s.wo, 0, 0, nullptr, 0, 0, 0,
+                dx, c * L, L, 1, 1.0f, rest, rest_bytes, stream, &cv);
 }
 
 int pam_hip_conv2d_fwd(const float* x, const float* w, float* y, long batch, long c, long h, long wd, long co, long kh, long kw,

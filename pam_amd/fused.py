@@ -149,10 +149,16 @@ def layer_norm(x, n, weight, bias, eps, offset=None, approx_bwd=False):
 
 # ---------------------------------------------------------------- convolution on image patches read in place
 
-def conv_in_place(X, W, dilation, approx_bwd):
+def input_gradient_in_place(W, stride, padding):
+    """The gradient of the input is a stride-1 convolution of the upstream gradient when the
+    forward stride is 1 and the padding does not exceed kernel - 1."""
+    return tuple(stride) == (1, 1) and padding[0] <= W.shape[2] - 1 and padding[1] <= W.shape[3] - 1
+
+
+def conv_in_place(X, W, dilation, approx_bwd, stride=(1, 1), padding=(0, 0)):
     """True when conv2d can run on the matrix kernel without unfolding X: fp32 GPU tensors,
-    dilation 1, and no exact gradient with respect to X wanted (that one needs the patches as
-    a stored operand)."""
+    dilation 1, and, if the exact gradient with respect to X is wanted, a geometry for which that
+    gradient is a convolution in place too (otherwise it needs the patches as a stored operand)."""
     if not (isinstance(X, torch.Tensor) and isinstance(W, torch.Tensor) and X.is_cuda and W.is_cuda):
         return False
     if X.dtype != torch.float32 or W.dtype != torch.float32 or X.dim() != 4 or W.dim() != 4 or X.numel() == 0:
@@ -160,7 +166,7 @@ def conv_in_place(X, W, dilation, approx_bwd):
     if dilation not in (1, (1, 1), [1, 1]):
         return False
     approx_x, _ = _both(approx_bwd)
-    return approx_x or not (torch.is_grad_enabled() and X.requires_grad)
+    return approx_x or not (torch.is_grad_enabled() and X.requires_grad) or input_gradient_in_place(W, stride, padding)
 
 
 class conv2d_autograd(torch.autograd.Function):
@@ -186,7 +192,9 @@ class conv2d_autograd(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             per_image = _abi.conv2d_bwd_weight(X, dY, W, ctx.stride, ctx.padding, not approx_w, off)
             dW = per_image.sum(0).view(W.shape)
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] and input_gradient_in_place(W, ctx.stride, ctx.padding):
+            dX = _abi.conv2d_bwd_input(dY, W, X, ctx.padding, not approx_x, off)
+        elif ctx.needs_input_grad[0]:
             if not approx_x:
                 raise RuntimeError("exact gradient with respect to the convolution input needs the unfolded path")
             batch, co = dY.shape[:2]

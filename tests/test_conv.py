@@ -79,33 +79,81 @@ def test_weight_gradient_against_oracle(oracle, case, off):
     assert_same_bits(got.cpu().numpy(), want, f"exact weight gradient {case}")
 
 
+STRIDE_ONE = [CASES[0], CASES[3], CASES[4],
+              (2, 5, 10, 13, 7, 3, 5, (1, 1), (2, 0)),        # padding k - 1 on one axis, none on the other
+              (1, 3, 6, 6, 4, 2, 2, (1, 1), (0, 0))]          # even kernel
+
+
+@pytest.mark.parametrize("off", [None, OFF])
+@pytest.mark.parametrize("case", STRIDE_ONE)
+def test_input_gradient_against_oracle(oracle, case, off):
+    """Stride 1: dX is the convolution of dY, padded by k - 1 - pad, with the flipped weights; the
+    oracle computes that product on the unfolded gradient with the library's accumulation plan."""
+    batch, c, h, w, co, kh, kw, stride, (ph, pw) = case
+    X, W = _inputs(case, 4)
+    ho, wo = h + 2 * ph - kh + 1, w + 2 * pw - kw + 1
+    rng = np.random.RandomState(5)
+    dY = (rng.standard_normal((batch, co, ho, wo)) * 1e-2).astype(np.float32)
+    dY.reshape(-1)[rng.choice(dY.size, max(2, dY.size // 50), replace=False)] = 0.0
+    P = torch.nn.functional.unfold(torch.from_numpy(dY), (kh, kw), padding=(kh - 1 - ph, kw - 1 - pw)).numpy()   # [B, co kh kw, h w]
+    K, L = P.shape[1:]
+    assert L == h * w
+    Wf = np.ascontiguousarray(W.transpose(1, 0, 2, 3)[:, :, ::-1, ::-1]).reshape(c, K)
+    plan = _plan(batch, c, L, K)
+    Xd, Wd, dYd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda(), torch.from_numpy(dY).cuda()
+    o = 1.0 if off is None else off
+    Wl = Wf if off is None else oracle.pam(Wf, np.float32(off))
+    want = oracle.gemm(np.broadcast_to(Wl, (batch, c, K)), P, kchunk=plan)
+    got = _abi.conv2d_bwd_input(dYd, Wd, Xd, (ph, pw), False, o)
+    assert_same_bits(got.cpu().numpy().reshape(batch, c, L), want, f"approximate input gradient {case}")
+    want = oracle.gemm(np.broadcast_to(Wf, (batch, c, K)), P, mode=oracle.MODE_BWD_DELTA_R, D=X.reshape(batch, c, L), offset=off, kchunk=plan)
+    got = _abi.conv2d_bwd_input(dYd, Wd, Xd, (ph, pw), True, o)
+    assert_same_bits(got.cpu().numpy().reshape(batch, c, L), want, f"exact input gradient {case}")
+
+
+def test_input_gradient_rejects_other_strides():
+    X = torch.randn(1, 2, 8, 8, device="cuda"); W = torch.randn(3, 2, 3, 3, device="cuda")
+    lib = _abi.load_library()
+    assert lib.pam_hip_conv2d_workspace_bytes(1, 2, 8, 8, 3, 3, 3, 2, 2, 1, 1, 2, 1.0) == 0
+    dY = torch.randn(1, 3, 4, 4, device="cuda"); dX = torch.empty_like(X); ws = torch.empty(1 << 16, device="cuda")
+    rc = lib.pam_hip_conv2d_bwd_input(dY.data_ptr(), W.data_ptr(), X.data_ptr(), dX.data_ptr(), 1, 2, 8, 8, 3, 3, 3, 2, 2, 1, 1,
+                                      0, 1.0, ws.data_ptr(), ws.numel() * 4, None)
+    assert rc == -1 and b"stride 1" in lib.pam_hip_last_error()
+    assert not pam_amd.fused.input_gradient_in_place(W, (2, 2), (1, 1)) and pam_amd.fused.input_gradient_in_place(W, (1, 1), (2, 2))
+    assert not pam_amd.fused.input_gradient_in_place(W, (1, 1), (3, 1))
+
+
 def _close(a, b, tol=3e-6):
     return (a - b).abs().max().item() <= tol * b.abs().max().item()
 
 
-@pytest.mark.parametrize("approx", [True, (True, False)])
-def test_module_path_matches_unfolded_composition(approx):
+@pytest.mark.parametrize("stride", [(2, 1), (1, 1)])
+@pytest.mark.parametrize("approx", [True, (True, False), False, (False, True)])
+def test_module_path_matches_unfolded_composition(approx, stride):
     """pam.conv2d / pam.Conv2d with patches read in place against the unfold + linear chain on the
-    same GPU: values and both gradients agree up to the grouping of the sums."""
+    same GPU: values and both gradients agree up to the grouping of the sums.  With stride 1 the
+    input gradient runs in place as well, the exact one included; with another stride the exact
+    input gradient sends the whole call down the unfolded path."""
     torch.manual_seed(0)
     X = torch.randn(4, 6, 14, 11, device="cuda"); W = torch.randn(10, 6, 3, 3, device="cuda") * 0.2; b = torch.randn(10, device="cuda")
-    g = torch.randn(4, 10, 7, 11, device="cuda")
+    g = torch.randn(4, 10, 7 if stride[0] == 2 else 14, 11, device="cuda")
     res = {}
     for implicit in (True, False):
         composites.implicit_conv = implicit
         try:
             Xr, Wr = X.clone().requires_grad_(), W.clone().requires_grad_()
-            Y = pam_amd.conv2d(Xr, Wr, b, stride=(2, 1), padding=1, offset=OFF, approx_bwd=approx)
+            Y = pam_amd.conv2d(Xr, Wr, b, stride=stride, padding=1, offset=OFF, approx_bwd=approx)
             Y.backward(g)
             res[implicit] = (Y.detach(), Xr.grad, Wr.grad)
         finally:
             composites.implicit_conv = True
-    assert res[True][0].is_contiguous()
+    in_place = stride == (1, 1) or approx is True or (isinstance(approx, tuple) and approx[0])
+    assert res[True][0].is_contiguous() == in_place
     for a, c in zip(res[True], res[False]):
         assert a.shape == c.shape and _close(a, c)
-    # an exact gradient with respect to the input keeps the unfolded path
+    # an exact gradient with respect to the input: in place for stride 1, else the unfolded path
     Xr = X.clone().requires_grad_()
-    pam_amd.conv2d(Xr, W, None, padding=1, approx_bwd=False).sum().backward()
+    pam_amd.conv2d(Xr, W, None, padding=1, stride=stride, approx_bwd=False).sum().backward()
     assert Xr.grad is not None and torch.isfinite(Xr.grad).all()
     # no gradient wanted for the input (first layer): in place whatever the flags
     Wr = W.clone().requires_grad_()
@@ -117,13 +165,18 @@ def test_conv_module_against_torch_on_exact_products():
     """Power-of-two weights make every PAM product exact (pam/test_pam.py:151-170): the layer equals F.conv2d."""
     torch.manual_seed(1)
     X1 = (torch.randint(-1024, 1024, (5, 13, 15, 17), device="cuda") / 64.0).requires_grad_()
-    conv = pam_amd.Conv2d(13, 19, (3, 5), padding=(1, 2), stride=(1, 2), approx_bwd=True).cuda()
+    _against_torch(X1, (1, 2))
+    _against_torch(X1.detach().clone().requires_grad_(), (1, 1))        # the input gradient in place
+
+
+def _against_torch(X1, stride):
+    conv = pam_amd.Conv2d(13, 19, (3, 5), padding=(1, 2), stride=stride, approx_bwd=True).cuda()
     with torch.no_grad():
         conv.weight.copy_(2.0 ** torch.randint(-8, 8, conv.weight.shape, device="cuda").float())
     X2 = X1.detach().clone().requires_grad_()
     Y1 = conv(X1); Y1.sum().backward()
-    Y2 = torch.nn.functional.conv2d(X2, conv.weight.detach(), conv.bias.detach(), padding=(1, 2), stride=(1, 2)); Y2.sum().backward()
+    Y2 = torch.nn.functional.conv2d(X2, conv.weight.detach(), conv.bias.detach(), padding=(1, 2), stride=stride); Y2.sum().backward()
     assert _close(Y1, Y2, 2e-6) and _close(X1.grad, X2.grad, 2e-6)
     Wt = conv.weight.detach().clone().requires_grad_()
-    torch.nn.functional.conv2d(X2.detach(), Wt, None, padding=(1, 2), stride=(1, 2)).sum().backward()
+    torch.nn.functional.conv2d(X2.detach(), Wt, None, padding=(1, 2), stride=stride).sum().backward()
     assert _close(conv.weight.grad, Wt.grad, 2e-6)
