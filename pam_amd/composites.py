@@ -5,9 +5,9 @@ additions, subtractions, maxima and sums are ordinary fp32 torch operations, as 
 reference.  Same names and keyword arguments.
 
 Reductions over the last dimension of a contiguous GPU tensor take the single-kernel path of
-`pam_amd.fused` (softmax always; logsumexp, log_softmax and layer_norm always for rows of up to
-1024 values, whose gradients are single kernels too, and otherwise, like mean, when no autograd
-graph is recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
+`pam_amd.fused` (softmax, logsumexp and log_softmax always, their gradients are single kernels too;
+layer_norm always for rows of up to 1024 values and otherwise, like mean, when no autograd graph is
+recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
 the single-kernel path off.  conv2d on GPU tensors runs on the matrix kernel with the image
 patches read in place instead of unfolded (`implicit_conv = False` switches that off).
 """

@@ -558,6 +558,74 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(CH >= 
     }
 }
 
+// The same gradient for rows too long for registers: two sweeps over the row in blocks of 64 x U
+// values (the second sweep finds the row in cache).  A lane meets its elements in the same ascending
+// order as in the register variant, so the sums are the same sums.
+template <class G>
+__device__ __forceinline__ void logsumexp_grad_stream(const float* __restrict__ xr, const float* __restrict__ gr, float* __restrict__ dr,
+                                                      float g_row, bool log_softmax, float shift, int lane, long n, G& m)
+{
+    constexpr int U = 8;
+    float p = 0.0f, q = 0.0f;
+    for (long base = 0; base < n; base += 64L * U) {
+        float xv[U], gy[U];
+#pragma unroll
+        for (int c = 0; c < U; ++c) {
+            const long i = base + lane + 64L * c; const bool inside = i < n;
+            xv[c] = inside ? xr[i] : 1.0f;
+            gy[c] = (inside && log_softmax) ? gr[i] : 0.0f;
+        }
+#pragma unroll
+        for (int c = 0; c < U; ++c) {
+            const bool inside = base + lane + 64L * c < n;
+            const float sc = m.mul(xv[c], kLog2E) - shift;
+            const float e = m.exp2(inside ? sc : 0.5f);
+            if (inside) { p = p + e; q = q + gy[c]; }
+        }
+    }
+    const float total = wave_sum(p);
+    const float g_out = log_softmax ? -wave_sum(q) : g_row;
+    const float u = shift + m.log2(total);
+    const float du = m.div_da(u, kLog2E, g_out);
+    const float dtotal = m.log2_dx(total, du);
+    for (long base = 0; base < n; base += 64L * U) {
+        float xv[U], gy[U];
+#pragma unroll
+        for (int c = 0; c < U; ++c) {
+            const long i = base + lane + 64L * c; const bool inside = i < n;
+            xv[c] = inside ? xr[i] : 1.0f;
+            gy[c] = (inside && log_softmax) ? gr[i] : 0.0f;
+        }
+#pragma unroll
+        for (int c = 0; c < U; ++c) {
+            const long i = base + lane + 64L * c; const bool inside = i < n;
+            const float sc = m.mul(xv[c], kLog2E) - shift;
+            const float d = m.mul_da(xv[c], kLog2E, m.exp2_dx(inside ? sc : 0.5f, dtotal));
+            if (inside) dr[i] = log_softmax ? gy[c] + d : d;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void logsumexp_bwd_stream_kernel(
+    const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
+    long rows, long n, int log_softmax, Offset o, Approx ap)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float shift = *shift_in;
+    for (long r = wave; r < rows; r += nwaves) {
+        const float* gr = log_softmax ? grad + r * n : nullptr;
+        const float g_row = log_softmax ? 0.0f : grad[r];
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            GradUnchecked u{o};
+            logsumexp_grad_stream(x + r * n, gr, dx + r * n, g_row, log_softmax != 0, shift, lane, n, u);
+            done = __ballot(!u.valid()) == 0ull;
+        }
+        if (!done) { GradChecked k{o, ap}; logsumexp_grad_stream(x + r * n, gr, dx + r * n, g_row, log_softmax != 0, shift, lane, n, k); }
+    }
+}
+
 // One row of the layer_norm gradient.  cen: x on entry, overwritten; g: dy on entry (1.0 past the
 // end), dx on exit; terms: the per-element terms of the weight gradient (if weight).
 template <int CH, class G>
@@ -792,10 +860,13 @@ int pam_hip_logsumexp_bwd(const float* x, const float* grad, const float* shift,
     if (rc != PAM_HIP_OK) return rc;
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !grad || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_bwd: null pointer");
-    if (n > 1024) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_bwd: rows of at most 1024 values");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    PAM_ROW_DISPATCH_REGS(logsumexp_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n,
-                          log_softmax, o, ap);
+    if (n > 1024)
+        hipLaunchKernelGGL(logsumexp_bwd_stream_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, grad, shift, dx,
+                           rows, n, log_softmax, o, ap);
+    else
+        PAM_ROW_DISPATCH_REGS(logsumexp_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n,
+                              log_softmax, o, ap);
     return pamhost::check_launch("logsumexp_bwd");
 }
 
