@@ -162,6 +162,9 @@ def main():
             ("pa_exp_fwd", 8, lambda: K.pa_exp_fwd(d, math.e, 1.0)), ("pa_log_fwd", 8, lambda: K.pa_log_fwd(a, math.e, 1.0)),
             ("pa_exp_bwd", 12, lambda: K.pa_exp_bwd(d, b, math.e, 1.0)), ("pa_log_bwd", 12, lambda: K.pa_log_bwd(a, b, math.e, 1.0)),
         )
+        from pam_amd import _abi as abi_ew
+        stream_ops += (("pow_0.5_fwd", 8, lambda: abi_ew.pow_fwd(a, 0.5, 1.0)),
+                       ("pow_0.5_bwd_approx", 12, lambda: abi_ew.pow_bwd(a, d, 0.5, 1.0, True, True)))
         for name, bpe, fn in stream_ops:
             ms = event_time_ms(fn, 10, torch)
             other[name] = {"ms": round(ms, 4), "GBps": round(bpe * n / ms / 1e6, 1), "hbm_frac": round(bpe * n / ms / 1e6 / 8000.0, 3)}

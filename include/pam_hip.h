@@ -202,6 +202,15 @@ int pam_hip_conv2d_bwd_input(const float *dy, const float *w, const float *x, fl
                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
                              int exact, float offset, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- power with a scalar exponent ---------------------------------------------------------- */
+/* y = x ** exponent = pa_exp2(pa_log2(x) (*) exponent), 0 where x is 0: the three elementwise
+ * launches and the select of pam.pow (pam/pam_ops.py:70-79) in one pass.  pow_bwd: the gradient for
+ * x that autograd chains through them (pam/cuda_bindings.py:43-57, 224-239, 262-276); approx_a
+ * selects the approximate gradient of the product, approx_exp that of exp2 and log2. */
+int pam_hip_pow_fwd(const float *x, float *y, size_t n, float exponent, float offset, void *stream);
+int pam_hip_pow_bwd(const float *x, const float *dy, float *dx, size_t n, float exponent, float offset,
+                    int approx_a, int approx_exp, void *stream);
+
 /* ---- optimizer step ---------------------------------------------------------------------- */
 /* One Adam update of n parameters in place, every product, the quotient and the square root
  * a PAM op                replaces the op-table arithmetic of the training recipe's optimizer

@@ -33,6 +33,8 @@ _SIGNATURES = {
     "pam_hip_pad_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
     "pam_hip_pa_exp_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_exp_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_pow_fwd": ([_p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_pow_bwd": ([_p, _p, _p, _z, _f, _f, _i, _i, _p], _i),
     "pam_hip_pa_log_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_log_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
     "pam_hip_gemm_workspace_bytes": ([_l, _l, _l, _l], _z),
@@ -373,6 +375,23 @@ class HipRowKernels:
                 _call("pam_hip_layer_norm_fwd", X.data_ptr(), None if weight is None else weight.data_ptr(),
                       None if bias is None else bias.data_ptr(), Y.data_ptr(), rows, n, float(eps), float(offset), _stream())
         return Y
+
+
+def pow_fwd(X, exponent, offset):
+    """X ** exponent (scalar) in one pass: exp2(log2(X) (*) exponent), zero where X is zero."""
+    return HipKernels._unary("pow_fwd", X, exponent, offset)
+
+
+def pow_bwd(X, dY, exponent, offset, approx_a, approx_exp):
+    """The gradient for X of pow_fwd, the chain through select, exp2, product and log2 in one pass."""
+    _check(X, dY)
+    out = torch.empty(X.shape, dtype=torch.float32, device=X.device)
+    if out.numel():
+        x, d = _flat(X), _flat(dY)
+        with torch.cuda.device(X.device):
+            _call("pam_hip_pow_bwd", x.data_ptr(), d.data_ptr(), out.data_ptr(), out.numel(), float(exponent), float(offset),
+                  int(bool(approx_a)), int(bool(approx_exp)), _stream())
+    return out
 
 
 def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, decay, step_size, offset):

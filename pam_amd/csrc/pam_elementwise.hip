@@ -67,6 +67,33 @@ struct OpLogBwd {   // (pam/cuda_kernels.cu:481-484); the inner pam_bwd runs wit
     }
 };
 
+// A ** p for a scalar exponent as the op library composes it: exp2(log2(A) (*) p), zero where A is
+// zero (pam/pam_ops.py:70-79), and the gradient for A that autograd chains from the three ops'
+// backward formulas (pam/cuda_bindings.py:43-57, 224-239, 262-276): through the select, exp2, the
+// product's first operand, log2.  ln 2 is math.log(2.0) rounded to fp32, as torch.full_like stores it.
+constexpr float kLn2 = (float)0.6931471805599453;
+struct OpPow {
+    float p, off; bool has_off;
+    __device__ float operator()(float a, float, float) const
+    {
+        if (a == 0.0f) return 0.0f;
+        return exp2_entry(pam_mul_off(log2_entry(a, off, has_off), p, off, has_off), off, has_off);
+    }
+};
+struct OpPowBwd {
+    float p, off; bool has_off, approx_a, approx_e;
+    __device__ float operator()(float a, float g, float) const
+    {
+        const float l = log2_entry(a, off, has_off);
+        const float t = pam_mul_off(l, p, off, has_off);
+        const float gy = a == 0.0f ? 0.0f : g;
+        const float gt = approx_e ? pam_mul_off(pam_mul_off(exp2_entry(t, off, has_off), kLn2, off, has_off), gy, off, has_off)
+                                  : exp2_entry_bwd(t, gy, off, has_off);
+        const float gl = approx_a ? pam_mul_off(gt, p, off, has_off) : pam_mul_bwd(l, p, gt, off, has_off);
+        return approx_e ? pad_div_off(pad_div_off(gl, a, off, has_off), kLn2, off, has_off) : log2_entry_bwd(a, gl, off, has_off);
+    }
+};
+
 template <class Op, int NIN>
 __global__ __launch_bounds__(kThreads) void ew_vec_kernel(const v4f* __restrict__ p0, const v4f* __restrict__ p1,
                                                          const v4f* __restrict__ p2, v4f* __restrict__ out,
@@ -265,6 +292,16 @@ int pam_hip_pa_exp_bwd(const float* x, const float* dy, float* dx, size_t n, flo
 
 int pam_hip_pa_log_bwd(const float* x, const float* dy, float* dx, size_t n, float base, float offset, void* stream)
 { return launch<OpLogBwd, 2>("pa_log_bwd", x, dy, nullptr, dx, n, OpLogBwd{log2f(base), offset, offset != 1.0f}, stream); }
+
+int pam_hip_pow_fwd(const float* x, float* y, size_t n, float exponent, float offset, void* stream)
+{ return launch<OpPow, 1>("pow_fwd", x, nullptr, nullptr, y, n, OpPow{exponent, offset, offset != 1.0f}, stream); }
+
+int pam_hip_pow_bwd(const float* x, const float* dy, float* dx, size_t n, float exponent, float offset,
+                    int approx_a, int approx_exp, void* stream)
+{
+    return launch<OpPowBwd, 2>("pow_bwd", x, dy, nullptr, dx, n,
+                               OpPowBwd{exponent, offset, offset != 1.0f, approx_a != 0, approx_exp != 0}, stream);
+}
 
 int pam_hip_adam_step(float* p, const float* g, float* m, float* v, size_t n, float beta1, float one_minus_beta1,
                       float beta2, float one_minus_beta2, float eps, float decay, int has_decay, float step_size,

@@ -147,6 +147,35 @@ def layer_norm(x, n, weight, bias, eps, offset=None, approx_bwd=False):
     return out.view(x.shape)
 
 
+# ---------------------------------------------------------------- power with a scalar exponent
+
+class pow_autograd(torch.autograd.Function):
+    """A ** p for a number p: log2, product, exp2 and the select of zeros (pam/pam_ops.py:70-79)
+    in one pass, and the gradient those ops' backward formulas chain to in another."""
+
+    @staticmethod
+    def forward(ctx, A, exponent, offset, approx_bwd):
+        ctx.exponent, ctx.offset, ctx.approx_bwd = float(exponent), _offset_value(offset), approx_bwd
+        ctx.save_for_backward(A)
+        return _abi.pow_fwd(A, ctx.exponent, ctx.offset)
+
+    @staticmethod
+    def backward(ctx, dY):
+        A, = ctx.saved_tensors
+        approx_a, _, approx_exp = _flags(ctx.approx_bwd)
+        return _abi.pow_bwd(A, dY.contiguous(), ctx.exponent, ctx.offset, approx_a, approx_exp), None, None, None
+
+
+def pow_in_place(A, B):
+    """fp32 GPU tensor to the power of a plain number."""
+    return (isinstance(A, torch.Tensor) and A.is_cuda and A.dtype == torch.float32
+            and isinstance(B, (int, float)) and not isinstance(B, bool))
+
+
+def pow_scalar(A, exponent, offset=None, approx_bwd=False):
+    return pow_autograd.apply(A, exponent, offset, approx_bwd)
+
+
 # ---------------------------------------------------------------- convolution on image patches read in place
 
 def input_gradient_in_place(W, stride, padding):

@@ -17,7 +17,7 @@ import yaml
 from . import _abi
 from .factories import get_function_dict
 
-__all__ = ["Adam"]
+__all__ = ["Adam", "multiply_grads"]
 
 
 def _pam_table_offset(cfg):
@@ -113,3 +113,19 @@ class Adam(torch.optim.Optimizer):
                 if half:
                     p.data.copy_(p32)
         return loss
+
+
+def multiply_grads(params, c, op_dict):
+    """The gradient-scaling hook of the reference's optimizer wrapper
+    (submodules/fairseq/fairseq/optim/fairseq_optimizer.py:103-119 in the reference tree): calls
+    op_dict['mul'](grad, c) for every dense gradient and, like the reference, drops the result (its
+    loop rebinds a local name), so dense gradients keep their values; sparse gradients are scaled in
+    place with an ordinary multiply.  Kept for callers that rely on exactly that behaviour."""
+    for p in params:
+        if p.grad is None:
+            continue
+        cc = c.to(p.grad.device) if torch.is_tensor(c) else c
+        if p.grad.is_sparse:
+            p.grad.data.mul_(cc)
+        else:
+            op_dict["mul"](p.grad.data, cc)

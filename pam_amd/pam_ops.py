@@ -17,6 +17,7 @@ from . import utils
 __all__ = ["mul", "div", "exp", "exp2", "log", "log2", "pow", "matmul", "bmm", "linear", "Linear"]
 
 fused_bias = True        # False: linear() adds the bias with a separate torch add, as the reference does
+fused_pow = True         # False: pow() with a number as exponent runs the chain of log2, product, exp2 and select
 
 
 def _require_kernel(t, use_kernel):
@@ -76,6 +77,8 @@ def log2(A, *, offset=None, approx_bwd=False, use_kernel=True):
 
 def pow(A, B, *, offset=None, approx_bwd=False, use_kernel=True):
     """A ** B as exp2(log2(A) (*) B), zero where A is zero (pam/pam_ops.py:70-79)."""
+    if fused_pow and use_kernel and fused.pow_in_place(A, B):
+        return fused.pow_scalar(A, B, offset, approx_bwd)             # one pass, and one for the gradient
     tA, tB = utils.to_tensor(A, B)
     kw = dict(offset=offset, approx_bwd=approx_bwd, use_kernel=use_kernel)
     out = torch.where(tA == 0, 0, exp2(mul(log2(tA, **kw), tB, **kw), **kw))

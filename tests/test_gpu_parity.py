@@ -476,3 +476,40 @@ def test_linear_with_bias_in_the_epilogue(oracle):
     ref = lin(x3)
     pam_ops.fused_bias = True
     assert torch.equal(lin(x3), ref) and lin(x3).shape == (4, 197, 96)
+
+
+@pytest.mark.parametrize("off", OFFS)
+@pytest.mark.parametrize("p", [0.5, 2.0, -1.5, 3])
+def test_pow_with_a_number_in_one_pass(K, oracle, p, off):
+    """pam.pow(A, number): one kernel against the reference's chain (pam/pam_ops.py:70-79) built from
+    the oracle's primitives, and against the same chain of kernels on the GPU -- values and the
+    gradient autograd chains through select, exp2, product and log2, bit for bit."""
+    import pam_amd
+    from pam_amd import pam_ops
+    rng = np.random.RandomState(17)
+    a = np.abs(rng.standard_normal(5003)).astype(np.float32) * 3 + 0.01
+    a[rng.choice(a.size, 40, replace=False)] = np.resize(np.array([0.0, -0.0, 1e-30, 1e30, 1.0, 2.0 ** -126, 1e-40, np.inf], np.float32), 40)
+    g = rng.standard_normal(a.shape).astype(np.float32)
+    l = oracle.pa_log(a, 2.0, off)
+    want = np.where(a == 0, np.float32(0), oracle.pa_exp(oracle.pam(l, np.float32(p), off), 2.0, off)).astype(np.float32)
+    res = {}
+    for fused_on in (True, False):
+        pam_ops.fused_pow = fused_on
+        try:
+            for approx in (False, True, (True, False), (False, True)):
+                at = dev(a).requires_grad_()
+                y = pam_amd.pow(at, p, offset=off, approx_bwd=approx)
+                y.backward(dev(g))
+                res[fused_on, approx] = (host(y.detach()), host(at.grad))
+        finally:
+            pam_ops.fused_pow = True
+    for approx in (False, True, (True, False), (False, True)):
+        assert_same_bits(res[True, approx][0], want, f"pow {p} forward")
+        assert_same_bits(res[True, approx][0], res[False, approx][0], f"pow {p}: one pass against the chain")
+        assert_same_bits(res[True, approx][1], res[False, approx][1], f"pow {p} gradient, approx={approx}: one pass against the chain")
+    # the exact gradient from the oracle's primitives
+    t = oracle.pam(l, np.float32(p), off)
+    gy = np.where(a == 0, np.float32(0), g).astype(np.float32)
+    gt = oracle.pa_exp_bwd(t, gy, 2.0, off)
+    gl = oracle.pam_bwd(l, np.full_like(l, p), gt, off)
+    assert_same_bits(res[True, False][1], oracle.pa_log_bwd(a, gl, 2.0, off), f"pow {p} exact gradient")

@@ -152,3 +152,13 @@ def test_gpu_optimizer_kernel_equals_op_by_op():
         results.append([p_.detach().cpu().numpy() for p_ in params] + [opt.state[p_]["exp_avg_sq"].cpu().numpy() for p_ in params])
     for a, b in zip(*results):
         assert_same_bits(a, b, "kernel vs op-by-op")
+
+
+def test_multiply_grads_keeps_dense_gradients_like_the_reference():
+    """fairseq_optimizer.py:103-119 computes mul(grad, c) and drops it; dense gradients stay as they are."""
+    from pam_amd.optim import multiply_grads
+    p = torch.nn.Parameter(torch.ones(4)); p.grad = torch.full((4,), 3.0)
+    q = torch.nn.Parameter(torch.ones(4))                      # no gradient
+    calls = []
+    multiply_grads([p, q], 0.5, {"mul": lambda a, b: calls.append((a.clone(), b)) or a * b})
+    assert len(calls) == 1 and calls[0][1] == 0.5 and torch.equal(p.grad, torch.full((4,), 3.0))
