@@ -112,8 +112,32 @@ def gemm_plan(batch, m, n, k):
     return c.value, g.value
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current device's current stream as a hipStream_t value."""
+    if _raw_stream is not None:                       # a plain integer, without building a Stream object
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+class _Current:
+    """Stands in for torch.cuda.device(d) when d already is the current device."""
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_CURRENT = _Current()
+
+
+def _on(device):
+    """Context that makes `device` current for the launches inside it."""
+    return _CURRENT if device.index is None or device.index == torch.cuda.current_device() else torch.cuda.device(device)
 
 
 def _check(*tensors):
@@ -148,7 +172,7 @@ class HipKernels:
         n = out.numel()
         if n == 0:
             return out
-        with torch.cuda.device(A.device):
+        with _on(A.device):
             if name in ("pam_fwd", "pad_fwd") and (_is_single_value(A) or _is_single_value(B)):
                 scalar_is_a = _is_single_value(A)
                 s, x = (A, B) if scalar_is_a else (B, A)
@@ -171,7 +195,7 @@ class HipKernels:
         n = out.numel()
         if n:
             a, b, d = _flat(A), _flat(B), _flat(dC)
-            with torch.cuda.device(A.device):
+            with _on(A.device):
                 _call(f"pam_hip_{name}", a.data_ptr(), b.data_ptr(), d.data_ptr(), out.data_ptr(), n, float(offset), _stream())
         return out
 
@@ -195,7 +219,7 @@ class HipKernels:
         n = out.numel()
         if n:
             x = _flat(X)
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 if dY is None:
                     _call(f"pam_hip_{name}", x.data_ptr(), out.data_ptr(), n, float(base), float(offset), _stream())
                 else:
@@ -237,7 +261,7 @@ class HipKernels:
         out = torch.empty((batch, m, n) if batched else (m, n), dtype=torch.float32, device=L.device)
         if out.numel() == 0:
             return out
-        with torch.cuda.device(L.device):
+        with _on(L.device):
             lib = load_library()
             ws_bytes = lib.pam_hip_gemm_workspace_bytes(batch, m, n, k)
             ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=L.device) if ws_bytes else None
@@ -296,7 +320,7 @@ class HipRowKernels:
         row_sum = torch.empty(rows, dtype=torch.float32, device=X.device)
         shift = torch.empty(1, dtype=torch.float32, device=X.device)
         if X.numel():
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 ws, nbytes = self._workspace(X.device)
                 _call("pam_hip_softmax_fwd", X.data_ptr(), Y.data_ptr(), row_sum.data_ptr(), shift.data_ptr(), rows, n,
                       float(offset), ws.data_ptr(), nbytes, _stream())
@@ -308,7 +332,7 @@ class HipRowKernels:
             raise ValueError("softmax_bwd: operand shapes do not match")
         dX = torch.empty_like(X)
         if X.numel():
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 _call("pam_hip_softmax_bwd", X.data_ptr(), dY.data_ptr(), row_sum.data_ptr(), shift.data_ptr(),
                       dX.data_ptr(), rows, n, float(offset), int(bool(approx_a)), int(bool(approx_b)),
                       int(bool(approx_exp)), _stream())
@@ -321,7 +345,7 @@ class HipRowKernels:
         Y = torch.empty_like(X) if want_log_softmax else None
         shift = torch.empty(1, dtype=torch.float32, device=X.device)
         if X.numel():
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 ws, nbytes = self._workspace(X.device)
                 _call("pam_hip_logsumexp_fwd", X.data_ptr(), lse.data_ptr() if want_lse else None,
                       Y.data_ptr() if want_log_softmax else None, shift.data_ptr(), rows, n, float(offset),
@@ -336,7 +360,7 @@ class HipRowKernels:
             raise ValueError("logsumexp_bwd: gradient has the wrong size")
         dX = torch.empty_like(X)
         if X.numel():
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 _call("pam_hip_logsumexp_bwd", X.data_ptr(), grad.data_ptr(), shift.data_ptr(), dX.data_ptr(), rows, n,
                       int(bool(log_softmax)), float(offset), int(bool(approx_a)), int(bool(approx_b)), int(bool(approx_exp)),
                       _stream())
@@ -350,7 +374,7 @@ class HipRowKernels:
         dX = torch.empty_like(X)
         terms = torch.empty_like(X) if (want_weight_terms and weight is not None) else None
         if X.numel():
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 _call("pam_hip_layer_norm_bwd", X.data_ptr(), None if weight is None else weight.data_ptr(), dY.data_ptr(),
                       dX.data_ptr(), None if terms is None else terms.data_ptr(), rows, n, float(eps), float(offset),
                       int(bool(approx_a)), int(bool(approx_b)), int(bool(approx_exp)), _stream())
@@ -360,7 +384,7 @@ class HipRowKernels:
         rows, n = self._rows("row_mean_fwd", X)
         Y = torch.empty(rows, dtype=torch.float32, device=X.device)
         if rows:
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 _call("pam_hip_row_mean_fwd", X.data_ptr(), Y.data_ptr(), rows, n, float(offset), _stream())
         return Y
 
@@ -371,7 +395,7 @@ class HipRowKernels:
                 raise ValueError("layer_norm_fwd: weight and bias must have one value per column")
         Y = torch.empty_like(X)
         if X.numel():
-            with torch.cuda.device(X.device):
+            with _on(X.device):
                 _call("pam_hip_layer_norm_fwd", X.data_ptr(), None if weight is None else weight.data_ptr(),
                       None if bias is None else bias.data_ptr(), Y.data_ptr(), rows, n, float(eps), float(offset), _stream())
         return Y
@@ -388,7 +412,7 @@ def pow_bwd(X, dY, exponent, offset, approx_a, approx_exp):
     out = torch.empty(X.shape, dtype=torch.float32, device=X.device)
     if out.numel():
         x, d = _flat(X), _flat(dY)
-        with torch.cuda.device(X.device):
+        with _on(X.device):
             _call("pam_hip_pow_bwd", x.data_ptr(), d.data_ptr(), out.data_ptr(), out.numel(), float(exponent), float(offset),
                   int(bool(approx_a)), int(bool(approx_exp)), _stream())
     return out
@@ -403,7 +427,7 @@ def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, d
     if not (p.shape == g.shape == m.shape == v.shape):
         raise ValueError("adam_step: tensors must have the same shape")
     if p.numel():
-        with torch.cuda.device(p.device):
+        with _on(p.device):
             _call("pam_hip_adam_step", p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel(), float(beta1),
                   float(one_minus_beta1), float(beta2), float(one_minus_beta2), float(eps), float(decay or 0.0),
                   int(bool(decay)), float(step_size), float(offset), _stream())
@@ -426,7 +450,7 @@ def conv2d_fwd(X, W, stride, padding, offset):
     ho, wo = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
     Y = torch.empty((batch, co, ho, wo), dtype=torch.float32, device=X.device)
     if Y.numel():
-        with torch.cuda.device(X.device):
+        with _on(X.device):
             nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 0, float(offset))
             ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=X.device)
             _call("pam_hip_conv2d_fwd", X.data_ptr(), W.data_ptr(), Y.data_ptr(), *geo, float(offset), ws.data_ptr(), nbytes, _stream())
@@ -441,7 +465,7 @@ def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset):
     batch, c, _, _, co, kh, kw = geo[:7]
     dW = torch.empty((batch, co, c * kh * kw), dtype=torch.float32, device=X.device)
     if dW.numel():
-        with torch.cuda.device(X.device):
+        with _on(X.device):
             nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 1, float(offset))
             ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=X.device)
             _call("pam_hip_conv2d_bwd_weight", X.data_ptr(), dY.data_ptr(), W.data_ptr(), dW.data_ptr(), *geo,
@@ -457,7 +481,7 @@ def conv2d_bwd_input(dY, W, X, padding, exact, offset):
     geo = _conv_geometry(X, W, (1, 1), padding)
     dX = torch.empty_like(X)
     if dX.numel():
-        with torch.cuda.device(X.device):
+        with _on(X.device):
             nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 2, float(offset))
             if nbytes == 0:
                 raise ValueError("conv2d_bwd_input: needs stride 1 and padding <= kernel - 1")
@@ -478,7 +502,7 @@ def linear_fwd(X, Wt, bias, offset):
         raise ValueError("linear_fwd: bias must be contiguous with one value per output column")
     out = torch.empty((m, n), dtype=torch.float32, device=X.device)
     if out.numel():
-        with torch.cuda.device(X.device):
+        with _on(X.device):
             ws_bytes = load_library().pam_hip_gemm_workspace_bytes(1, m, n, k)
             ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
             _call("pam_hip_pam_linear_fwd", X.data_ptr(), X.stride(0), X.stride(1), Wt.data_ptr(), Wt.stride(0), Wt.stride(1),

@@ -462,8 +462,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 
 // ---------------------------------------------------------------- gradients of logsumexp / log_softmax and layer_norm
 // Autograd's chain over the unfused ops, written out (pam/cuda_bindings.py:43-57, 78-97, 224-239,
-// 262-276 for the formulas; pam/pam_ops.py:331-378 for the ops).  Register-resident rows only
-// (n <= 1024).  GradChecked serves every combination of exact and approximate gradients;
+// 262-276 for the formulas; pam/pam_ops.py:331-378 for the ops).  Rows of up to 1024 values stay in
+// registers; beyond that logsumexp / log_softmax sweep the row twice and layer_norm is not served.
+// GradChecked serves every combination of exact and approximate gradients;
 // GradUnchecked is the all-approximate chain on the branch-free primitives, tried first and kept
 // when every value it touched was a normal number.
 struct GradChecked {
