@@ -483,10 +483,10 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                 for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
             }
         } else if (verdict == kZerosL && MODE == MODE_PAM) {
-#pragma unroll 2
+#pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) zeros_left_step(kk);
         } else if (verdict == kZerosR && MODE == MODE_PAM) {
-#pragma unroll 2
+#pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) zeros_right_step(kk);
         } else if (verdict == (kZerosL | kZerosR) && MODE == MODE_PAM) {
 #pragma unroll 2

@@ -27,6 +27,12 @@ namespace {
 #ifndef PAM_ROW_WAVES
 #define PAM_ROW_WAVES 4
 #endif
+#ifndef PAM_ROW_WAVES_SHORT
+#define PAM_ROW_WAVES_SHORT 8
+#endif
+// rows of up to 256 values need few registers: more wavefronts in flight hide the load latency of the short rows
+#define PAM_ROW_OCC(CH) (((CH) > 0 && (CH) <= 4) ? PAM_ROW_WAVES_SHORT : PAM_ROW_WAVES)
+#define PAM_ROW_OCC_GRAD(CH) ((CH) >= 16 ? 2 : PAM_ROW_OCC(CH))
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 constexpr int kMaxPartials = 1024;
@@ -200,7 +206,7 @@ __device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)
 }
 
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC(CH)))) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                               float* __restrict__ row_sum, float* __restrict__ shift_out,
                                                               long rows, long n, Offset o,
                                                               const float* __restrict__ partial, int partials)
@@ -288,7 +294,7 @@ __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], c
 }
 
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC(CH)))) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                               const float* __restrict__ row_sum, const float* __restrict__ shift_in,
                                                               float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
 {
@@ -350,7 +356,7 @@ __device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shif
 }
 
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC(CH)))) void logsumexp_kernel(const float* __restrict__ x, float* __restrict__ lse,
                                                             float* __restrict__ y, float* __restrict__ shift_out, long rows, long n,
                                                             Offset o, const float* __restrict__ partial, int partials)
 {
@@ -433,7 +439,7 @@ __device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&ou
 }
 
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void layer_norm_fwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC(CH)))) void layer_norm_fwd_kernel(const float* __restrict__ x, const float* __restrict__ weight,
                                                                  const float* __restrict__ bias, float* __restrict__ y,
                                                                  long rows, long n, float eps, Offset o)
 {
@@ -533,7 +539,7 @@ __device__ __forceinline__ void logsumexp_grad_row(const float (&xv)[CH], const 
 
 // dx of out = logsumexp(x) (per row, gradient g_out) or of y = x - logsumexp(x) (gradient gy per element)
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(CH >= 16 ? 2 : PAM_ROW_WAVES))) void logsumexp_bwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC_GRAD(CH)))) void logsumexp_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
     long rows, long n, int log_softmax, Offset o, Approx ap)
 {
@@ -683,7 +689,7 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
 
 // dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(CH >= 16 ? 2 : PAM_ROW_WAVES))) void layer_norm_bwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >= 16 ? 2 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
     float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
 {
