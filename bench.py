@@ -168,6 +168,9 @@ def main():
         a_pos = a.abs()                                                   # a square root's operand (edge values stay)
         stream_ops += (("pow_0.5_fwd", 8, lambda: abi_ew.pow_fwd(a_pos, 0.5, 1.0)),
                        ("pow_0.5_bwd_approx", 12, lambda: abi_ew.pow_bwd(a_pos, d, 0.5, 1.0, True, True)))
+        stream_ops += (("pam_bwd_pair_approx", 20, lambda: K.pam_bwd_pair(a, b, d, 1.0, True, True)),
+                       ("pam_bwd_pair_exact", 20, lambda: K.pam_bwd_pair(a, b, d, 1.0, False, False)),
+                       ("pad_bwd_pair_approx", 20, lambda: K.pad_bwd_pair(a, b, d, 1.0, True, True)))
         for name, bpe, fn in stream_ops:
             ms = event_time_ms(fn, 30, torch)
             other[name] = {"ms": round(ms, 4), "GBps": round(bpe * n / ms / 1e6, 1), "hbm_frac": round(bpe * n / ms / 1e6 / 8000.0, 3)}

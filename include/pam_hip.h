@@ -55,6 +55,16 @@ int pam_hip_pad_fwd(const float *a, const float *b, float *c, size_t n, float of
 /* dB = d/dB (A (/) B) * dC            replaces pad_bwd  (elementwise_pad_bwd_caller, :296-328) */
 int pam_hip_pad_bwd(const float *a, const float *b, const float *dc, float *db, size_t n, float offset, void *stream);
 
+/* Both gradients of C = A (*) B or C = A (/) B in one pass over A, B, dC (20 B per element), the
+ * formulas of the reference's autograd functions (pam/cuda_bindings.py:43-57, 78-97), which run two
+ * to six elementwise launches for them: approx_x != 0 selects the approximate gradient of that
+ * operand (product: dC (*) other; quotient: (1 (/) B) (*) dC and -((A (/) B) (/) B) (*) dC), else
+ * the exact one (pam_bwd / pad_bwd above; for the quotient's dA, pam_bwd(A, 1 (/) B, dC) without offset). */
+int pam_hip_pam_bwd_pair(const float *a, const float *b, const float *dc, float *da, float *db, size_t n, float offset,
+                         int approx_a, int approx_b, void *stream);
+int pam_hip_pad_bwd_pair(const float *a, const float *b, const float *dc, float *da, float *db, size_t n, float offset,
+                         int approx_a, int approx_b, void *stream);
+
 /* Variants of the two forward ops with one operand a single fp32 value in device memory
  * (the reference materialises broadcast scalars with flatten(), pam/cuda_kernels.cu:163-164;
  * these read 8 B/element instead of 12).  scalar_is_a != 0: C = s[0] (op) X, else C = X (op) s[0]. */

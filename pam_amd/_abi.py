@@ -33,6 +33,8 @@ _SIGNATURES = {
     "pam_hip_pad_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
     "pam_hip_pa_exp_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_exp_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_pam_bwd_pair": ([_p, _p, _p, _p, _p, _z, _f, _i, _i, _p], _i),
+    "pam_hip_pad_bwd_pair": ([_p, _p, _p, _p, _p, _z, _f, _i, _i, _p], _i),
     "pam_hip_pow_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pow_bwd": ([_p, _p, _p, _z, _f, _f, _i, _i, _p], _i),
     "pam_hip_pa_log_fwd": ([_p, _p, _z, _f, _f, _p], _i),
@@ -207,6 +209,28 @@ class HipKernels:
 
     def pam_bwd(self, A, B, dC, offset):
         return self._ternary("pam_bwd", A, B, dC, offset)
+
+    @staticmethod
+    def _pair(name, A, B, dC, offset, approx_a, approx_b):
+        _check(A, B, dC)
+        if not (A.shape == B.shape == dC.shape):
+            raise ValueError(f"{name}: operands must have the same shape")
+        dA = torch.empty(A.shape, dtype=torch.float32, device=A.device)
+        dB = torch.empty(A.shape, dtype=torch.float32, device=A.device)
+        if dA.numel():
+            a, b, d = _flat(A), _flat(B), _flat(dC)
+            with _on(A.device):
+                _call(f"pam_hip_{name}", a.data_ptr(), b.data_ptr(), d.data_ptr(), dA.data_ptr(), dB.data_ptr(), dA.numel(),
+                      float(offset), int(bool(approx_a)), int(bool(approx_b)), _stream())
+        return dA, dB
+
+    def pam_bwd_pair(self, A, B, dC, offset, approx_a, approx_b):
+        """(dA, dB) of C = A (*) B in one pass; not part of the reference's extension surface."""
+        return self._pair("pam_bwd_pair", A, B, dC, offset, approx_a, approx_b)
+
+    def pad_bwd_pair(self, A, B, dC, offset, approx_a, approx_b):
+        """(dA, dB) of C = A (/) B in one pass; not part of the reference's extension surface."""
+        return self._pair("pad_bwd_pair", A, B, dC, offset, approx_a, approx_b)
 
     def pad_bwd(self, A, B, dC, offset):
         return self._ternary("pad_bwd", A, B, dC, offset)

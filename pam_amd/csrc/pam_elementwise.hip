@@ -162,6 +162,91 @@ int launch(const char* what, const float* p0, const float* p1, const float* p2, 
     return pamhost::check_launch(what);
 }
 
+// ---------------------------------------------------------------- both gradients of a product / quotient in one pass
+// autograd asks for dA and dB of C = A (*) B or A (/) B together; the reference computes them with two
+// to six launches (pam/cuda_bindings.py:43-57, 78-97).  Same formulas per element, one read of A, B, dC.
+struct PairPam {
+    float off; bool has_off, approx_a, approx_b;
+    __device__ void operator()(float a, float b, float d, float& da, float& db) const
+    {
+        da = approx_a ? pam_mul_off(d, b, off, has_off) : pam_mul_bwd(a, b, d, off, has_off);
+        db = approx_b ? pam_mul_off(d, a, off, has_off) : pam_mul_bwd(b, a, d, off, has_off);
+    }
+};
+struct PairPad {
+    float off; bool has_off, approx_a, approx_b;
+    __device__ void operator()(float a, float b, float d, float& da, float& db) const
+    {
+        const float inv = pad_div_off(1.0f, b, off, has_off);
+        da = approx_a ? pam_mul_off(inv, d, off, has_off) : pam_mul_bwd(a, inv, d, 1.0f, false);
+        db = approx_b ? -pam_mul_off(pad_div_off(pad_div_off(a, b, off, has_off), b, off, has_off), d, off, has_off)
+                      : pad_div_bwd(a, b, d, off, has_off);
+    }
+};
+
+template <class Op>
+__global__ __launch_bounds__(kThreads) void pair_vec_kernel(const v4f* __restrict__ pa, const v4f* __restrict__ pb, const v4f* __restrict__ pd,
+                                                           v4f* __restrict__ oa, v4f* __restrict__ ob, size_t nvec, Op op)
+{
+    constexpr int U = 2;
+    const size_t step = (size_t)gridDim.x * (kThreads * U);
+    for (size_t base = (size_t)blockIdx.x * (kThreads * U) + threadIdx.x; base < nvec; base += step) {
+        v4f a[U], b[U], d[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            size_t i = base + (size_t)u * kThreads;
+            if (i < nvec) { a[u] = __builtin_nontemporal_load(pa + i); b[u] = __builtin_nontemporal_load(pb + i); d[u] = __builtin_nontemporal_load(pd + i); }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            size_t i = base + (size_t)u * kThreads;
+            if (i < nvec) {
+                v4f ra, rb; float x, y;
+                op(a[u].x, b[u].x, d[u].x, x, y); ra.x = x; rb.x = y;
+                op(a[u].y, b[u].y, d[u].y, x, y); ra.y = x; rb.y = y;
+                op(a[u].z, b[u].z, d[u].z, x, y); ra.z = x; rb.z = y;
+                op(a[u].w, b[u].w, d[u].w, x, y); ra.w = x; rb.w = y;
+                __builtin_nontemporal_store(ra, oa + i); __builtin_nontemporal_store(rb, ob + i);
+            }
+        }
+    }
+}
+
+template <class Op>
+__global__ __launch_bounds__(kThreads) void pair_scalar_kernel(const float* __restrict__ pa, const float* __restrict__ pb, const float* __restrict__ pd,
+                                                              float* __restrict__ oa, float* __restrict__ ob, size_t first, size_t n, Op op)
+{
+    const size_t step = (size_t)gridDim.x * kThreads;
+    for (size_t i = first + (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += step) {
+        float x, y;
+        op(pa[i], pb[i], pd[i], x, y);
+        oa[i] = x; ob[i] = y;
+    }
+}
+
+template <class Op>
+int launch_pair(const char* what, const float* a, const float* b, const float* d, float* da, float* db, size_t n, Op op, void* stream)
+{
+    if (n == 0) return PAM_HIP_OK;
+    if (!a || !b || !d || !da || !db) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: null pointer", what);
+    hipStream_t st = (hipStream_t)stream;
+    uintptr_t align = (uintptr_t)a | (uintptr_t)b | (uintptr_t)d | (uintptr_t)da | (uintptr_t)db;
+    size_t nvec = (align & 15u) ? 0 : n / 4;
+    const size_t cap = (size_t)1 << 30;
+    if (nvec) {
+        size_t blocks = (nvec + kThreads * 2 - 1) / (kThreads * 2);
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(pair_vec_kernel<Op>, dim3((unsigned)blocks), dim3(kThreads), 0, st,
+                           (const v4f*)a, (const v4f*)b, (const v4f*)d, (v4f*)da, (v4f*)db, nvec, op);
+    }
+    if (nvec * 4 < n) {
+        size_t blocks = (n - nvec * 4 + kThreads - 1) / kThreads;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(pair_scalar_kernel<Op>, dim3((unsigned)blocks), dim3(kThreads), 0, st, a, b, d, da, db, nvec * 4, n, op);
+    }
+    return pamhost::check_launch(what);
+}
+
 // ---------------------------------------------------------------- Adam step
 // One update of a parameter tensor by the Adam variant whose products, quotient and square
 // root are PAM ops (the training recipe's optimizer, fairseq/optim/adam.py:226-252 in the
@@ -262,6 +347,14 @@ int pam_hip_pam_bwd(const float* a, const float* b, const float* dc, float* da, 
 
 int pam_hip_pad_bwd(const float* a, const float* b, const float* dc, float* db, size_t n, float offset, void* stream)
 { return launch<OpPadBwd, 3>("pad_bwd", a, b, dc, db, n, OpPadBwd{offset, offset != 1.0f}, stream); }
+
+int pam_hip_pam_bwd_pair(const float* a, const float* b, const float* dc, float* da, float* db, size_t n, float offset,
+                         int approx_a, int approx_b, void* stream)
+{ return launch_pair("pam_bwd_pair", a, b, dc, da, db, n, PairPam{offset, offset != 1.0f, approx_a != 0, approx_b != 0}, stream); }
+
+int pam_hip_pad_bwd_pair(const float* a, const float* b, const float* dc, float* da, float* db, size_t n, float offset,
+                         int approx_a, int approx_b, void* stream)
+{ return launch_pair("pad_bwd_pair", a, b, dc, da, db, n, PairPad{offset, offset != 1.0f, approx_a != 0, approx_b != 0}, stream); }
 
 int pam_hip_pam_fwd_bcast(const float* x, const float* s, int scalar_is_a, float* c, size_t n, float offset, void* stream)
 {

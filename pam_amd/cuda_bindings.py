@@ -28,6 +28,15 @@ def _both(approx_bwd):
     return (approx_bwd, approx_bwd) if isinstance(approx_bwd, bool) else tuple(approx_bwd)
 
 
+paired_gradients = True      # False: one launch per gradient, as the reference's autograd functions do
+
+
+def _pair_kernel(k, name, A, B):
+    """Both gradients in one pass when the kernel object has that entry point and neither operand is a
+    broadcast view (flattening it would materialise the copy the single-gradient path avoids)."""
+    return paired_gradients and hasattr(k, name) and A.is_contiguous() and B.is_contiguous()
+
+
 class pam_autograd(torch.autograd.Function):
     """C = A (*) B elementwise (pam/cuda_bindings.py:27-57)."""
 
@@ -44,9 +53,15 @@ class pam_autograd(torch.autograd.Function):
         k, off = cuda_kernels, ctx.offset
         approx_A, approx_B = _both(ctx.approx_bwd)
         dY = delta_Y.contiguous()
+        need_A, need_B = ctx.needs_input_grad[:2]
+        if need_A and need_B and _pair_kernel(k, "pam_bwd_pair", A, B):
+            return (*k.pam_bwd_pair(A, B, dY, off, approx_A, approx_B), None, None)
         # approximate: treat PAM as a product, d/dA = B; exact: the slope of the affine piece
-        delta_A = k.pam_fwd(dY, B, off) if approx_A else k.pam_bwd(A, B, dY, off)
-        delta_B = k.pam_fwd(dY, A, off) if approx_B else k.pam_bwd(B, A, dY, off)
+        delta_A = delta_B = None
+        if need_A:
+            delta_A = k.pam_fwd(dY, B, off) if approx_A else k.pam_bwd(A, B, dY, off)
+        if need_B:
+            delta_B = k.pam_fwd(dY, A, off) if approx_B else k.pam_bwd(B, A, dY, off)
         return delta_A, delta_B, None, None
 
 
@@ -71,18 +86,23 @@ class pad_autograd(torch.autograd.Function):
         k, off = cuda_kernels, ctx.offset
         approx_A, approx_B = _both(ctx.approx_bwd)
         dY = delta_Y.contiguous()
+        need_A, need_B = ctx.needs_input_grad[:2]
+        if need_A and need_B and _pair_kernel(k, "pad_bwd_pair", A, B):
+            return (*k.pad_bwd_pair(A, B, dY, off, approx_A, approx_B), None, None)
 
-        inv_B = k.pad_fwd(torch.ones_like(B), B, off)            # 1 (/) B
-        if approx_A:
-            delta_A = k.pam_fwd(inv_B, dY, off)
-        else:
-            delta_A = k.pam_bwd(A, inv_B, dY, 1.0)
-
-        if approx_B:
-            slope = k.pad_fwd(k.pad_fwd(A, B, off), B, off)      # (A (/) B) (/) B
-            delta_B = -k.pam_fwd(slope, dY, off)
-        else:
-            delta_B = k.pad_bwd(A, B, dY, off)
+        delta_A = delta_B = None
+        if need_A:
+            inv_B = k.pad_fwd(torch.ones_like(B), B, off)        # 1 (/) B
+            if approx_A:
+                delta_A = k.pam_fwd(inv_B, dY, off)
+            else:
+                delta_A = k.pam_bwd(A, inv_B, dY, 1.0)
+        if need_B:
+            if approx_B:
+                slope = k.pad_fwd(k.pad_fwd(A, B, off), B, off)  # (A (/) B) (/) B
+                delta_B = -k.pam_fwd(slope, dY, off)
+            else:
+                delta_B = k.pad_bwd(A, B, dY, off)
         return delta_A, delta_B, None, None
 
 

@@ -513,3 +513,40 @@ def test_pow_with_a_number_in_one_pass(K, oracle, p, off):
     gt = oracle.pa_exp_bwd(t, gy, 2.0, off)
     gl = oracle.pam_bwd(l, np.full_like(l, p), gt, off)
     assert_same_bits(res[True, False][1], oracle.pa_log_bwd(a, gl, 2.0, off), f"pow {p} exact gradient")
+
+
+@pytest.mark.parametrize("off", OFFS)
+def test_both_gradients_in_one_pass(K, oracle, off):
+    """(dA, dB) of a product / quotient from one kernel against the oracle's formulas
+    (pam/cuda_bindings.py:43-57, 78-97) and, through autograd, against the one-launch-per-gradient path."""
+    import pam_amd
+    from pam_amd import cuda_bindings
+    n = 10007
+    a, b, d = _rand((n,), 51, 0.01, True), _rand((n,), 52, 0.01, True), _rand((n,), 53, 0.01, True)
+    o = _o(off)
+    inv = oracle.pad(np.ones_like(b), b, off)
+    want = {
+        ("pam", True): (oracle.pam(d, b, off), oracle.pam(d, a, off)),
+        ("pam", False): (oracle.pam_bwd(a, b, d, off), oracle.pam_bwd(b, a, d, off)),
+        ("pad", True): (oracle.pam(inv, d, off), -oracle.pam(oracle.pad(oracle.pad(a, b, off), b, off), d, off)),
+        ("pad", False): (oracle.pam_bwd(a, inv, d, None), oracle.pad_bwd(a, b, d, off)),
+    }
+    for op in ("pam", "pad"):
+        for approx_a in (True, False):
+            for approx_b in (True, False):
+                da, db = getattr(K, f"{op}_bwd_pair")(dev(a), dev(b), dev(d), o, approx_a, approx_b)
+                assert_same_bits(host(da), want[op, approx_a][0], f"{op} dA approx={approx_a}")
+                assert_same_bits(host(db), want[op, approx_b][1], f"{op} dB approx={approx_b}")
+    # through autograd: paired against single launches, unaligned views included
+    for fn in (pam_amd.mul, pam_amd.div):
+        res = {}
+        for paired in (True, False):
+            cuda_bindings.paired_gradients = paired
+            try:
+                at, bt = dev(a)[1:].requires_grad_(), dev(b)[1:].requires_grad_()
+                fn(at, bt, offset=off, approx_bwd=(True, False)).backward(dev(d)[1:])
+                res[paired] = (host(at.grad), host(bt.grad))
+            finally:
+                cuda_bindings.paired_gradients = True
+        assert_same_bits(res[True][0], res[False][0], "dA paired against single")
+        assert_same_bits(res[True][1], res[False][1], "dB paired against single")
