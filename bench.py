@@ -165,9 +165,9 @@ def main():
             ("pa_exp_bwd", 12, lambda: K.pa_exp_bwd(d, b, math.e, 1.0)), ("pa_log_bwd", 12, lambda: K.pa_log_bwd(a, b, math.e, 1.0)),
         )
         from pam_amd import _abi as abi_ew
-        a_pos = a.abs()                                                   # a square root's operand (edge values stay)
-        stream_ops += (("pow_0.5_fwd", 8, lambda: abi_ew.pow_fwd(a_pos, 0.5, 1.0)),
-                       ("pow_0.5_bwd_approx", 12, lambda: abi_ew.pow_bwd(a_pos, d, 0.5, 1.0, True, True)))
+        a_pos = torch.randn(n, generator=g).to(dev).abs_().add_(1e-3)     # a square root's operand: positive normal numbers
+        stream_ops += (("pow_0.5_fwd_positive_operand", 8, lambda: abi_ew.pow_fwd(a_pos, 0.5, 1.0)),
+                       ("pow_0.5_bwd_approx_positive_operand", 12, lambda: abi_ew.pow_bwd(a_pos, d, 0.5, 1.0, True, True)))
         stream_ops += (("pam_bwd_pair_approx", 20, lambda: K.pam_bwd_pair(a, b, d, 1.0, True, True)),
                        ("pam_bwd_pair_exact", 20, lambda: K.pam_bwd_pair(a, b, d, 1.0, False, False)),
                        ("pad_bwd_pair_approx", 20, lambda: K.pad_bwd_pair(a, b, d, 1.0, True, True)))

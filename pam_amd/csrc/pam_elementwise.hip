@@ -79,6 +79,13 @@ struct OpPow {
         if (a == 0.0f) return 0.0f;
         return exp2_entry(pam_mul_off(log2_entry(a, off, has_off), p, off, has_off), off, has_off);
     }
+    // branch-free form, exact whenever every value it touches is a normal number and a > 0 (else redone checked)
+    __device__ bool has_fast() const { return true; }
+    __device__ float fast(float a, float, float, Span& sp) const
+    {
+        sp.in_exp_range = sp.in_exp_range && a > 0.0f;
+        return exp2_entry_unchecked(pam_unchecked_off(log2_entry_unchecked(a, off, has_off, sp), p, off, has_off, sp), off, has_off, sp);
+    }
 };
 struct OpPowBwd {
     float p, off; bool has_off, approx_a, approx_e;
@@ -92,7 +99,22 @@ struct OpPowBwd {
         const float gl = approx_a ? pam_mul_off(gt, p, off, has_off) : pam_mul_bwd(l, p, gt, off, has_off);
         return approx_e ? pad_div_off(pad_div_off(gl, a, off, has_off), kLn2, off, has_off) : log2_entry_bwd(a, gl, off, has_off);
     }
+    __device__ bool has_fast() const { return approx_a && approx_e; }       // the all-approximate chain
+    __device__ float fast(float a, float g, float, Span& sp) const
+    {
+        sp.in_exp_range = sp.in_exp_range && a > 0.0f;
+        const float l = log2_entry_unchecked(a, off, has_off, sp);
+        const float t = pam_unchecked_off(l, p, off, has_off, sp);
+        const float y = exp2_entry_unchecked(t, off, has_off, sp);
+        const float gt = pam_unchecked_off(pam_unchecked_off(y, kLn2, off, has_off, sp), g, off, has_off, sp);
+        const float gl = pam_unchecked_off(gt, p, off, has_off, sp);
+        return pad_unchecked_off(pad_unchecked_off(gl, a, off, has_off, sp), kLn2, off, has_off, sp);
+    }
 };
+
+// ops that also have a branch-free form `fast(a, b, c, Span&)`
+template <class Op, class = void> struct HasFast { static constexpr bool value = false; };
+template <class Op> struct HasFast<Op, decltype((void)&Op::has_fast)> { static constexpr bool value = true; };
 
 template <class Op, int NIN>
 __global__ __launch_bounds__(kThreads) void ew_vec_kernel(const v4f* __restrict__ p0, const v4f* __restrict__ p1,
@@ -116,10 +138,23 @@ __global__ __launch_bounds__(kThreads) void ew_vec_kernel(const v4f* __restrict_
             size_t i = base + (size_t)u * kThreads;
             if (i < nvec) {
                 v4f r;
-                r.x = op(a[u].x, NIN > 1 ? b[u].x : 0.f, NIN > 2 ? c[u].x : 0.f);
-                r.y = op(a[u].y, NIN > 1 ? b[u].y : 0.f, NIN > 2 ? c[u].y : 0.f);
-                r.z = op(a[u].z, NIN > 1 ? b[u].z : 0.f, NIN > 2 ? c[u].z : 0.f);
-                r.w = op(a[u].w, NIN > 1 ? b[u].w : 0.f, NIN > 2 ? c[u].w : 0.f);
+                bool done = false;
+                if constexpr (HasFast<Op>::value) {
+                    if (op.has_fast()) {
+                        Span sp;
+                        r.x = op.fast(a[u].x, NIN > 1 ? b[u].x : 0.f, NIN > 2 ? c[u].x : 0.f, sp);
+                        r.y = op.fast(a[u].y, NIN > 1 ? b[u].y : 0.f, NIN > 2 ? c[u].y : 0.f, sp);
+                        r.z = op.fast(a[u].z, NIN > 1 ? b[u].z : 0.f, NIN > 2 ? c[u].z : 0.f, sp);
+                        r.w = op.fast(a[u].w, NIN > 1 ? b[u].w : 0.f, NIN > 2 ? c[u].w : 0.f, sp);
+                        done = sp.normal();
+                    }
+                }
+                if (!done) {
+                    r.x = op(a[u].x, NIN > 1 ? b[u].x : 0.f, NIN > 2 ? c[u].x : 0.f);
+                    r.y = op(a[u].y, NIN > 1 ? b[u].y : 0.f, NIN > 2 ? c[u].y : 0.f);
+                    r.z = op(a[u].z, NIN > 1 ? b[u].z : 0.f, NIN > 2 ? c[u].z : 0.f);
+                    r.w = op(a[u].w, NIN > 1 ? b[u].w : 0.f, NIN > 2 ? c[u].w : 0.f);
+                }
                 __builtin_nontemporal_store(r, out + i);
             }
         }
