@@ -39,6 +39,8 @@
 //  * Accumulation order: every output is summed by one lane per k chunk, k ascending, from
 //    +0 -- with one chunk this is the order of the reference kernel
 //    (pam/cuda_kernels.cu:601, 608-627); pam_hip_gemm_plan reports the chunking.
+#include <cmath>
+
 #include "pam_common.h"
 #include "pam_device.h"
 
@@ -619,9 +621,20 @@ Plan make_plan(long batch, long M, long N, long K, bool allow_split)
     long maxsplit = kunits / 4;                                  // at least 128 k per work-group
     if (want > maxsplit) want = maxsplit;
     if (allow_split && want > 1) {
-        long per = (kunits + want - 1) / want;
-        p.kchunk = (int)(per * KGRAN);
-        p.ksplit = (int)((kunits + per - 1) / per);
+        // Work-groups are dealt to the compute units in rounds of one each, and a round that is nearly empty costs
+        // almost a full one: of the split counts next to the wanted one, take the one whose last round is fullest
+        // (each extra chunk also costs a little in the reduction).
+        long best_per = 0; double best = 0.0;
+        for (long w = want - 1; w <= want + 1; ++w) {
+            if (w < 2 || w > maxsplit || (g_force_ksplit > 0 && w != want)) continue;
+            const long per = (kunits + w - 1) / w, chunks = (kunits + per - 1) / per;
+            const double rounds = (double)(tiles * chunks) / (double)cus;
+            const double cost = std::ceil(rounds) / rounds * (1.0 + 0.015 * (double)chunks);
+            if (best_per == 0 || cost < best) { best = cost; best_per = per; }
+        }
+        if (best_per == 0) best_per = (kunits + want - 1) / want;
+        p.kchunk = (int)(best_per * KGRAN);
+        p.ksplit = (int)((kunits + best_per - 1) / best_per);
     }
     return p;
 }
