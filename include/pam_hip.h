@@ -167,8 +167,8 @@ int pam_hip_row_mean_fwd(const float *x, float *y, long rows, long n, float offs
 int pam_hip_layer_norm_fwd(const float *x, const float *weight, const float *bias, float *y, long rows, long n,
                            float eps, float offset, void *stream);
 /* Gradients of the two above, the chain autograd runs over the unfused ops
- * (pam/cuda_bindings.py:43-57, 78-97, 224-239, 262-276) in one kernel each; layer_norm_bwd takes
- * rows of at most 1024 values (an argument error beyond), logsumexp_bwd any length.
+ * (pam/cuda_bindings.py:43-57, 78-97, 224-239, 262-276) in one kernel each, for rows of any length
+ * (up to 1024 values a row stays in registers, longer rows are swept several times).
  * logsumexp_bwd: grad is [rows] (log_softmax == 0) or [rows][n] (the gradient of x - logsumexp(x));
  * shift is the forward's global shift.  layer_norm_bwd: dw_terms[rows][n], if not NULL, receives
  * the per-element terms whose sum over rows is the weight gradient (the bias gradient is the sum

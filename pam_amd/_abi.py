@@ -376,7 +376,6 @@ class HipRowKernels:
                       ws.data_ptr(), nbytes, _stream())
         return lse, Y, shift
 
-    max_grad_row = 1024          # the layer_norm gradient kernel keeps a row in registers
 
     def logsumexp_bwd(self, X, grad, shift, offset, approx_a, approx_b, approx_exp, log_softmax):
         rows, n = self._rows("logsumexp_bwd", X, grad, shift)

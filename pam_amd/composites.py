@@ -5,9 +5,8 @@ additions, subtractions, maxima and sums are ordinary fp32 torch operations, as 
 reference.  Same names and keyword arguments.
 
 Reductions over the last dimension of a contiguous GPU tensor take the single-kernel path of
-`pam_amd.fused` (softmax, logsumexp and log_softmax always, their gradients are single kernels too;
-layer_norm always for rows of up to 1024 values and otherwise, like mean, when no autograd graph is
-recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
+`pam_amd.fused` (softmax, logsumexp, log_softmax and layer_norm always, their gradients are single
+kernels too; mean when no autograd graph is recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
 the single-kernel path off.  conv2d on GPU tensors runs on the matrix kernel with the image
 patches read in place instead of unfolded (`implicit_conv = False` switches that off).
 """
@@ -77,7 +76,7 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
     """pam/pam_ops.py:331-342; inputs must be finite."""
     kw = _pam_kwargs(offset, approx_bwd, use_kernel)
     assert x.isfinite().all()
-    if _fused(x, dim, use_kernel, x, kernel_gradient=fused.has_gradient_kernel(x)):
+    if _fused(x, dim, use_kernel, x):
         return fused.logsumexp(x, keepdim, offset, approx_bwd)
     weights, shift = _scaled_exp2(x, kw, None)
     total = torch.sum(weights, dim=dim, keepdim=keepdim)
@@ -86,7 +85,7 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
 
 def log_softmax(x, dim=None, *, offset=None, approx_bwd=False, use_kernel=True):
     """pam/pam_ops.py:345-347"""
-    if _fused(x, dim, use_kernel, x, kernel_gradient=fused.has_gradient_kernel(x)):
+    if _fused(x, dim, use_kernel, x):
         assert x.isfinite().all()
         return fused.log_softmax(x, offset, approx_bwd)
     return x - logsumexp(x, dim=dim, keepdim=True, **_pam_kwargs(offset, approx_bwd, use_kernel))
@@ -100,7 +99,7 @@ def layer_norm(x, normalized_shape, weight=None, bias=None, eps=1e-05, *,
     if isinstance(normalized_shape, int):
         normalized_shape = (normalized_shape,)
     assert x.shape[-len(normalized_shape):] == normalized_shape
-    if _fused(x, -1, use_kernel, x, weight, bias, kernel_gradient=math.prod(normalized_shape) <= 1024) and all(
+    if _fused(x, -1, use_kernel, x, weight, bias) and all(
             t is None or (t.is_cuda and t.dtype == torch.float32) for t in (weight, bias)):
         return fused.layer_norm(x, math.prod(normalized_shape), weight, bias, eps, offset, approx_bwd)
     rows = x.reshape((-1, math.prod(normalized_shape)))

@@ -469,7 +469,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 // ---------------------------------------------------------------- gradients of logsumexp / log_softmax and layer_norm
 // Autograd's chain over the unfused ops, written out (pam/cuda_bindings.py:43-57, 78-97, 224-239,
 // 262-276 for the formulas; pam/pam_ops.py:331-378 for the ops).  Rows of up to 1024 values stay in
-// registers; beyond that logsumexp / log_softmax sweep the row twice and layer_norm is not served.
+// registers; longer rows are swept several times (the later sweeps find the row in cache).
 // GradChecked serves every combination of exact and approximate gradients;
 // GradUnchecked is the all-approximate chain on the branch-free primitives, tried first and kept
 // when every value it touched was a normal number.
@@ -687,6 +687,81 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
     for (int c = 0; c < CH; ++c) g[c] = g[c] + ds1;
 }
 
+// The same gradient for rows too long for registers: five sweeps over the row (sum, sum of squares, the
+// denominator's gradient, the centred values' gradients and their sum, the final add); after the first sweep
+// the row comes from cache.  A lane meets its elements in the same ascending order as in the register
+// variant, so the three row sums are the same sums.  dx holds the centred values' gradients between the
+// last two sweeps (each lane re-reads only what it wrote itself).
+template <class G>
+__device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__ xr, const float* __restrict__ gr,
+                                                       const float* __restrict__ weight, float* __restrict__ dr,
+                                                       float* __restrict__ tr, int lane, long n, float count, float eps, G& m)
+{
+    float p = 0.0f;
+    for (long i = lane; i < n; i += 64) p = p + xr[i];
+    const float s1 = wave_sum(p);
+    const float mu = m.div(s1, count);
+    p = 0.0f;
+    for (long i = lane; i < n; i += 64) { const float c = xr[i] - mu; p = p + m.mul(c, c); }
+    const float s2 = wave_sum(p);
+    const float v = m.div(s2, count) + eps;
+    const float lg = m.log2(v);
+    const float half = m.mul(lg, 0.5f);
+    const float root = m.exp2(half);
+    const float denom = v == 0.0f ? 0.0f : root;
+    // the upstream gradient behind the weight product (and that product's term for the weight gradient)
+    auto behind_weight = [&](long i, float c, bool store_term) {
+        float g = gr[i];
+        if (weight) {
+            const float xn = m.div(c, denom), wi = weight[i];
+            if (store_term && tr) tr[i] = m.mul_db(xn, wi, g);
+            g = m.mul_da(xn, wi, g);
+        }
+        return g;
+    };
+    p = 0.0f;
+    for (long i = lane; i < n; i += 64) {
+        const float c = xr[i] - mu;
+        p = p + m.div_db(c, denom, behind_weight(i, c, true));
+    }
+    float d = wave_sum(p);
+    if (v == 0.0f) d = 0.0f;
+    d = m.exp2_dx(half, d);
+    d = m.mul_da(lg, 0.5f, d);
+    d = m.log2_dx(v, d);
+    const float ds2 = m.div_da(s2, count, d);
+    p = 0.0f;
+    for (long i = lane; i < n; i += 64) {
+        const float c = xr[i] - mu;
+        float dc = m.div_da(c, denom, behind_weight(i, c, false));
+        dc = dc + m.mul_da(c, c, ds2);
+        dc = dc + m.mul_db(c, c, ds2);
+        dr[i] = dc;
+        p = p + dc;
+    }
+    const float ds1 = m.div_da(s1, count, -wave_sum(p));
+    for (long i = lane; i < n; i += 64) dr[i] = dr[i] + ds1;
+}
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void layer_norm_bwd_stream_kernel(
+    const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
+    float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
+{
+    const int lane = threadIdx.x % 64;
+    const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
+    const float count = (float)n;
+    for (long r = wave; r < rows; r += nwaves) {
+        float* tr = (weight && dw_terms) ? dw_terms + r * n : nullptr;
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            GradUnchecked u{o};
+            layer_norm_grad_stream(x + r * n, gy + r * n, weight, dx + r * n, tr, lane, n, count, eps, u);
+            done = __ballot(!u.valid()) == 0ull;
+        }
+        if (!done) { GradChecked k{o, ap}; layer_norm_grad_stream(x + r * n, gy + r * n, weight, dx + r * n, tr, lane, n, count, eps, k); }
+    }
+}
+
 // dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias
 template <int CH>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >= 16 ? 2 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
@@ -884,10 +959,13 @@ int pam_hip_layer_norm_bwd(const float* x, const float* weight, const float* dy,
     if (rc != PAM_HIP_OK) return rc;
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !dy || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_bwd: null pointer");
-    if (n > 1024) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_bwd: rows of at most 1024 values");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    PAM_ROW_DISPATCH_REGS(layer_norm_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms,
-                          rows, n, eps, o, ap);
+    if (n > 1024)
+        hipLaunchKernelGGL(layer_norm_bwd_stream_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, weight, dy, dx,
+                           dw_terms, rows, n, eps, o, ap);
+    else
+        PAM_ROW_DISPATCH_REGS(layer_norm_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms,
+                              rows, n, eps, o, ap);
     return pamhost::check_launch("layer_norm_bwd");
 }
 

@@ -68,11 +68,6 @@ def _flags(approx_bwd):
     return a, b, bool(approx_bwd)
 
 
-def has_gradient_kernel(x, layer_norm=False):
-    """logsumexp and log_softmax have a gradient kernel for any row length; layer_norm's keeps a row in registers."""
-    return not layer_norm or x.shape[-1] <= row_kernels.max_grad_row
-
-
 def needs_graph(*tensors):
     return _wants_grad(*tensors)
 
