@@ -6,7 +6,7 @@ reference.  Same names and keyword arguments.
 
 Reductions over the last dimension of a contiguous GPU tensor take the single-kernel path of
 `pam_amd.fused` (softmax, logsumexp, log_softmax and layer_norm always, their gradients are single
-kernels too; mean when no autograd graph is recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
+kernels too; mean with the approximate gradient, or when no autograd graph is recorded); every other call runs the chain of primitive kernels written out below.  `fused_rows = False` switches
 the single-kernel path off.  conv2d on GPU tensors runs on the matrix kernel with the image
 patches read in place instead of unfolded (`implicit_conv = False` switches that off).
 """
@@ -43,7 +43,7 @@ def mean(input, dim=None, keepdim=False, *, dtype=None, offset=None, approx_bwd=
         dim = tuple(range(input.dim()))
     elif isinstance(dim, int):
         dim = (dim,)
-    if dtype in (None, torch.float32) and _fused(input, dim, use_kernel, input, kernel_gradient=False):
+    if dtype in (None, torch.float32) and _fused(input, dim, use_kernel, input, kernel_gradient=fused.mean_gradient_in_place(approx_bwd)):
         return fused.mean_last(input, keepdim, offset)
     count = math.prod(input.shape[d] for d in dim)
     total = torch.sum(input, dim=dim, keepdim=keepdim, dtype=dtype)

@@ -104,8 +104,32 @@ def log_softmax(x, offset=None, approx_bwd=False):
     return logsumexp_autograd.apply(x.reshape(-1, x.shape[-1]), offset, approx_bwd, True, True).view(x.shape)
 
 
+class mean_autograd(torch.autograd.Function):
+    """Row mean = (fixed-order row sum) (/) n with the approximate gradient of the quotient
+    (pam/cuda_bindings.py:86-87): every element of a row receives (1 (/) n) (*) g."""
+
+    @staticmethod
+    def forward(ctx, rows, offset):
+        ctx.offset, ctx.n = _offset_value(offset), rows.shape[1]
+        return row_kernels.row_mean_fwd(rows, ctx.offset)
+
+    @staticmethod
+    def backward(ctx, g):
+        k = cuda_bindings.cuda_kernels
+        g = g.contiguous().view(-1)
+        count = torch.full((1,), float(ctx.n), dtype=torch.float32, device=g.device).expand_as(g)
+        inv = k.pad_fwd(torch.ones((1,), dtype=torch.float32, device=g.device).expand_as(g), count, ctx.offset)
+        return k.pam_fwd(inv, g, ctx.offset).unsqueeze(1).expand(-1, ctx.n), None
+
+
+def mean_gradient_in_place(approx_bwd):
+    """The single-kernel mean carries the approximate gradient only (the exact one needs the row sum as the
+    forward pass rounded it)."""
+    return bool(_both(approx_bwd)[0])
+
+
 def mean_last(x, keepdim, offset=None):
-    y = row_kernels.row_mean_fwd(x.reshape(-1, x.shape[-1]), _offset_value(offset))
+    y = mean_autograd.apply(x.reshape(-1, x.shape[-1]), offset)
     return y.view(x.shape[:-1] + ((1,) if keepdim else ()))
 
 

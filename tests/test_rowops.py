@@ -396,3 +396,30 @@ def test_gpu_row_gradients_match_unfused_composition():
     wide = _dev(rows_case(42, 3, 1500, masks=False)).requires_grad_()
     pam_amd.layer_norm(wide, 1500, approx_bwd=True).sum().backward()
     assert torch.isfinite(wide.grad).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("off", [None, OFF])
+def test_gpu_mean_gradient(oracle, off):
+    """mean over the last dimension in training: the single kernel's approximate gradient is the chain's,
+    (1 (/) n) (*) g for every element, bit for bit; the exact gradient keeps the chain."""
+    x = rows_case(77, 37, 300, masks=False)
+    g = np.random.RandomState(8).standard_normal(37).astype(np.float32)
+    res = {}
+    for fused_on in (True, False):
+        composites.fused_rows = fused_on
+        try:
+            xt = _dev(x).requires_grad_()
+            y = pam_amd.mean(xt, dim=-1, offset=off, approx_bwd=True)
+            y.backward(_dev(g))
+            res[fused_on] = (y.detach().cpu().numpy(), xt.grad.cpu().numpy())
+        finally:
+            composites.fused_rows = True
+    assert_same_bits(res[True][0], oracle.row_mean_fwd(x, off), "mean")
+    assert np.abs(res[True][0] - res[False][0]).max() <= 1e-6 * np.abs(res[False][0]).max() + 1e-7      # torch.sum's order
+    assert_same_bits(res[True][1], res[False][1], "mean gradient against the chain")
+    want = oracle.pam(oracle.pad(np.ones_like(g), np.full_like(g, 300.0), off), g, off)
+    assert_same_bits(res[True][1], np.broadcast_to(want[:, None], x.shape), "mean gradient")
+    xt = _dev(x).requires_grad_()
+    pam_amd.mean(xt, dim=-1, offset=off, approx_bwd=False).backward(_dev(g))                             # exact: the chain
+    assert torch.isfinite(xt.grad).all()
