@@ -255,3 +255,13 @@ def test_kernel_object_rejects_host_tensors():
         k.pam_fwd(x, x, 1.0)
     with pytest.raises(RuntimeError, match="CUDA tensor"):
         k.pam_matmul_fwd(x, x, True, True, 1.0)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU; asking for more ends with a message instead of a silent single-GPU run."""
+    import pathlib
+    import subprocess
+    import sys
+    root = pathlib.Path(__file__).resolve().parents[1]
+    res = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0 and "one GPU" in res.stderr and res.stdout.strip() == ""
