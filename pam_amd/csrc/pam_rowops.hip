@@ -698,10 +698,12 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
                                                        float* __restrict__ tr, int lane, long n, float count, float eps, G& m)
 {
     float p = 0.0f;
+#pragma unroll 4
     for (long i = lane; i < n; i += 64) p = p + xr[i];
     const float s1 = wave_sum(p);
     const float mu = m.div(s1, count);
     p = 0.0f;
+#pragma unroll 4
     for (long i = lane; i < n; i += 64) { const float c = xr[i] - mu; p = p + m.mul(c, c); }
     const float s2 = wave_sum(p);
     const float v = m.div(s2, count) + eps;
@@ -720,6 +722,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
         return g;
     };
     p = 0.0f;
+#pragma unroll 4
     for (long i = lane; i < n; i += 64) {
         const float c = xr[i] - mu;
         p = p + m.div_db(c, denom, behind_weight(i, c, true));
@@ -731,6 +734,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
     d = m.log2_dx(v, d);
     const float ds2 = m.div_da(s2, count, d);
     p = 0.0f;
+#pragma unroll 4
     for (long i = lane; i < n; i += 64) {
         const float c = xr[i] - mu;
         float dc = m.div_da(c, denom, behind_weight(i, c, false));
@@ -740,6 +744,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
         p = p + dc;
     }
     const float ds1 = m.div_da(s1, count, -wave_sum(p));
+#pragma unroll 4
     for (long i = lane; i < n; i += 64) dr[i] = dr[i] + ds1;
 }
 
