@@ -182,21 +182,24 @@ int pam_hip_layer_norm_bwd(const float *x, const float *weight, const float *dy,
 /* The reference computes conv2d as unfold -> transpose copy -> PAM linear, a kh*kw-fold copy of
  * the input.  These entry points run the same products and sums on the matrix kernel with the
  * image patches read in place: x[batch][c][h][w] and w[co][c][kh][kw] contiguous, dilation 1,
- * output size (in + 2 pad - k) / stride + 1.  Sums run over k = (c, i, j) in ascending order in
- * the chunks pam_hip_gemm_plan(batch, co, ho*wo, c*kh*kw) reports. */
+ * output size (in + 2 pad - k) / stride + 1.  groups > 1 is the grouped convolution of
+ * pam.conv2d_group (:163-198): w[co][c / groups][kh][kw], channels and filters fall into groups that
+ * do not mix, one product per group on the same kernel (groups = 1 otherwise).  Sums run over
+ * k = (c, i, j) of the group in ascending order in the chunks
+ * pam_hip_gemm_plan(batch, co / groups, ho*wo, (c / groups)*kh*kw) reports. */
 size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
-                                      long stride_h, long stride_w, long pad_h, long pad_w, int which, float offset);
+                                      long stride_h, long stride_w, long pad_h, long pad_w, long groups, int which, float offset);
 /* which: 0 forward, 1 weight gradient, 2 input gradient */
 /* y[batch][co][ho][wo] = sum_k x_patch (*) (w (*) offset)           replaces pam.conv2d's forward */
 int pam_hip_conv2d_fwd(const float *x, const float *w, float *y, long batch, long c, long h, long wd, long co, long kh, long kw,
-                       long stride_h, long stride_w, long pad_h, long pad_w, float offset,
+                       long stride_h, long stride_w, long pad_h, long pad_w, long groups, float offset,
                        void *workspace, size_t workspace_bytes, void *stream);
 /* dw[batch][co][c*kh*kw]: each image's contribution to the weight gradient (the caller sums over
  * the batch, as autograd does for the reference's broadcast weight).  exact == 0: the
  * approximate gradient sum_l x_patch (*) (dy (*) offset) (pam/cuda_bindings.py:160-161);
  * exact != 0: sum_l pam_bwd(w, x_patch, dy) (:162-164), w required. */
 int pam_hip_conv2d_bwd_weight(const float *x, const float *dy, const float *w, float *dw, long batch, long c, long h, long wd,
-                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w, long groups,
                               int exact, float offset, void *workspace, size_t workspace_bytes, void *stream);
 
 /* dx[batch][c][h][w] for stride 1 (any other stride is an argument error: the caller keeps the
@@ -209,7 +212,7 @@ int pam_hip_conv2d_bwd_weight(const float *x, const float *dy, const float *w, f
  * Sums run over k = (co, i, j) ascending in the chunks pam_hip_gemm_plan(batch, c, h*w, co*kh*kw)
  * reports; the reference's order is that of its matrix kernel followed by torch's fold. */
 int pam_hip_conv2d_bwd_input(const float *dy, const float *w, const float *x, float *dx, long batch, long c, long h, long wd,
-                             long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                             long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w, long groups,
                              int exact, float offset, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- power with a scalar exponent ---------------------------------------------------------- */

@@ -48,10 +48,10 @@ _SIGNATURES = {
     "pam_hip_standard_bmm": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_matmul_bwd": (_MAT2 * 4 + [_l, _l, _l, _i, _f, _p, _z, _p], _i),
     "pam_hip_pam_bmm_bwd": (_MAT * 4 + [_l, _l, _l, _l, _i, _f, _p, _z, _p], _i),
-    "pam_hip_conv2d_workspace_bytes": ([_l] * 11 + [_i, _f], _z),
-    "pam_hip_conv2d_fwd": ([_p, _p, _p] + [_l] * 11 + [_f, _p, _z, _p], _i),
-    "pam_hip_conv2d_bwd_weight": ([_p, _p, _p, _p] + [_l] * 11 + [_i, _f, _p, _z, _p], _i),
-    "pam_hip_conv2d_bwd_input": ([_p, _p, _p, _p] + [_l] * 11 + [_i, _f, _p, _z, _p], _i),
+    "pam_hip_conv2d_workspace_bytes": ([_l] * 12 + [_i, _f], _z),
+    "pam_hip_conv2d_fwd": ([_p, _p, _p] + [_l] * 12 + [_f, _p, _z, _p], _i),
+    "pam_hip_conv2d_bwd_weight": ([_p, _p, _p, _p] + [_l] * 12 + [_i, _f, _p, _z, _p], _i),
+    "pam_hip_conv2d_bwd_input": ([_p, _p, _p, _p] + [_l] * 12 + [_i, _f, _p, _z, _p], _i),
     "pam_hip_adam_step": ([_p, _p, _p, _p, _z, _f, _f, _f, _f, _f, _f, _i, _f, _f, _p], _i),
     "pam_hip_rowop_workspace_bytes": ([], _z),
     "pam_hip_softmax_fwd": ([_p, _p, _p, _p, _l, _l, _f, _p, _z, _p], _i),
@@ -456,20 +456,20 @@ def adam_step(p, g, m, v, beta1, one_minus_beta1, beta2, one_minus_beta2, eps, d
                   int(bool(decay)), float(step_size), float(offset), _stream())
 
 
-def _conv_geometry(X, W, stride, padding):
-    if X.dim() != 4 or W.dim() != 4 or X.shape[1] != W.shape[1]:
-        raise ValueError("conv2d: expected X[batch, c, h, w] and W[co, c, kh, kw]")
+def _conv_geometry(X, W, stride, padding, groups=1):
+    if X.dim() != 4 or W.dim() != 4 or groups < 1 or X.shape[1] != W.shape[1] * groups or W.shape[0] % groups:
+        raise ValueError("conv2d: expected X[batch, c, h, w] and W[co, c / groups, kh, kw]")
     batch, c, h, w = X.shape
     co, _, kh, kw = W.shape
-    return [batch, c, h, w, co, kh, kw, stride[0], stride[1], padding[0], padding[1]]
+    return [batch, c, h, w, co, kh, kw, stride[0], stride[1], padding[0], padding[1], groups]
 
 
-def conv2d_fwd(X, W, stride, padding, offset):
+def conv2d_fwd(X, W, stride, padding, offset, groups=1):
     """Y[batch, co, ho, wo] for contiguous fp32 GPU tensors, dilation 1; the image patches are read in place."""
     _check(X, W)
     X, W = X.contiguous(), W.contiguous()
-    geo = _conv_geometry(X, W, stride, padding)
-    batch, c, h, w, co, kh, kw, sh, sw, ph, pw = geo
+    geo = _conv_geometry(X, W, stride, padding, groups)
+    batch, c, h, w, co, kh, kw, sh, sw, ph, pw, _ = geo
     ho, wo = (h + 2 * ph - kh) // sh + 1, (w + 2 * pw - kw) // sw + 1
     Y = torch.empty((batch, co, ho, wo), dtype=torch.float32, device=X.device)
     if Y.numel():
@@ -480,13 +480,13 @@ def conv2d_fwd(X, W, stride, padding, offset):
     return Y
 
 
-def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset):
-    """Per-image weight gradients [batch, co, c*kh*kw]; W is only read by the exact variant."""
+def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset, groups=1):
+    """Per-image weight gradients [batch, co, (c / groups)*kh*kw]; W is only read by the exact variant."""
     _check(X, dY, W)
     X, dY, W = X.contiguous(), dY.contiguous(), W.contiguous()
-    geo = _conv_geometry(X, W, stride, padding)
+    geo = _conv_geometry(X, W, stride, padding, groups)
     batch, c, _, _, co, kh, kw = geo[:7]
-    dW = torch.empty((batch, co, c * kh * kw), dtype=torch.float32, device=X.device)
+    dW = torch.empty((batch, co, c // groups * kh * kw), dtype=torch.float32, device=X.device)
     if dW.numel():
         with _on(X.device):
             nbytes = load_library().pam_hip_conv2d_workspace_bytes(*geo, 1, float(offset))
@@ -496,12 +496,12 @@ def conv2d_bwd_weight(X, dY, W, stride, padding, exact, offset):
     return dW
 
 
-def conv2d_bwd_input(dY, W, X, padding, exact, offset):
+def conv2d_bwd_input(dY, W, X, padding, exact, offset, groups=1):
     """dX[batch, c, h, w] of a stride-1 convolution with dY's patches read in place; X gives the
     shape and, for the exact variant, the values."""
     _check(dY, W, X)
     dY, W, X = dY.contiguous(), W.contiguous(), X.contiguous()
-    geo = _conv_geometry(X, W, (1, 1), padding)
+    geo = _conv_geometry(X, W, (1, 1), padding, groups)
     dX = torch.empty_like(X)
     if dX.numel():
         with _on(X.device):

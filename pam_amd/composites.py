@@ -177,10 +177,15 @@ def conv2d(X, W, bias=None, stride=1, padding=0, dilation=1, *, offset=None, app
 
 def conv2d_group(X, W, bias=None, stride=1, padding=0, dilation=1, groups=1, *,
                  offset=None, approx_bwd=False, use_kernel=True):
-    """Grouped convolution as unfold + one PAM bmm over the groups (pam/pam_ops.py:163-198)."""
+    """Grouped convolution (pam/pam_ops.py:163-198: unfold + one PAM bmm over the groups); on the matrix kernel
+    with the patches read in place where `fused.conv_in_place` allows."""
     batch, c_in = X.shape[:2]
     c_out, _, kh, kw = W.shape
     padding, stride, (h_out, w_out) = _conv_geometry(X.shape[2:], (kh, kw), stride, padding)
+    if implicit_conv and use_kernel and c_in % groups == 0 and c_out % groups == 0 and fused.conv_in_place(
+            X, W, dilation, approx_bwd, stride, padding, groups):
+        out = fused.conv2d(X, W, stride, padding, offset, approx_bwd, groups)        # patches read in place, one product per group
+        return out if bias is None else out + bias.view((1, -1, 1, 1))
     per_group = c_in // groups * kh * kw
     patches = torch.nn.functional.unfold(X, kernel_size=(kh, kw), padding=padding, stride=stride, dilation=dilation)
     patches = patches.view(batch, groups, per_group, -1).permute(1, 2, 0, 3).reshape(groups, per_group, -1)

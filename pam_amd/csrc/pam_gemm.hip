@@ -724,7 +724,13 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
 }
 
 // ---------------------------------------------------------------- convolution as a product with image patches
-struct ConvShape { long batch, c, h, w, co, kh, kw, sh, sw, ph, pw, ho, wo; long K() const { return c * kh * kw; } long L() const { return ho * wo; } };
+// groups: channels and filters fall into `g` groups that do not mix (weights [co][c / g][kh][kw]); K() is the
+// length of one group's sums
+struct ConvShape {
+    long batch, c, h, w, co, kh, kw, sh, sw, ph, pw, ho, wo, g;
+    long cg() const { return c / g; } long cog() const { return co / g; }
+    long K() const { return cg() * kh * kw; } long L() const { return ho * wo; }
+};
 
 __global__ __launch_bounds__(256) void conv_tables_kernel(int2* __restrict__ ktab, int2* __restrict__ ltab, int K, int L,
                                                          int kh, int kw, int H, int W, int wo, int sh, int sw, int ph, int pw)
@@ -747,13 +753,15 @@ __global__ __launch_bounds__(256) void scale_kernel(const float* __restrict__ in
 
 // wf[c][co][i][j] = w[co][c][kh-1-i][kw-1-j] (*) off: the weights of the convolution over the
 // upstream gradient that yields the gradient of the input (stride 1)
-__global__ __launch_bounds__(256) void flip_weights_kernel(const float* __restrict__ w, float* __restrict__ wf, int c, int co, int kh, int kw,
+// (with groups: c runs over all channels, co over the filters of c's group, and w is [filters][c per group][kh][kw])
+__global__ __launch_bounds__(256) void flip_weights_kernel(const float* __restrict__ w, float* __restrict__ wf, int c, int cog, int cg, int kh, int kw,
                                                           float off, int has_off)
 {
     const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= c * co * kh * kw) return;
-    const int j = idx % kw, i = (idx / kw) % kh, o = (idx / (kw * kh)) % co, ci = idx / (kw * kh * co);
-    const float v = w[(((long)o * c + ci) * kh + (kh - 1 - i)) * kw + (kw - 1 - j)];
+    if (idx >= c * cog * kh * kw) return;
+    const int j = idx % kw, i = (idx / kw) % kh, o = (idx / (kw * kh)) % cog, ci = idx / (kw * kh * cog);
+    const int filter = (ci / cg) * cog + o;
+    const float v = w[(((long)filter * cg + ci % cg) * kh + (kh - 1 - i)) * kw + (kw - 1 - j)];
     wf[idx] = has_off ? pam_mul(v, off) : v;
 }
 
@@ -763,6 +771,8 @@ int conv_shape(const char* what, ConvShape& s)
 {
     if (s.batch < 0 || s.c <= 0 || s.h <= 0 || s.w <= 0 || s.co <= 0 || s.kh <= 0 || s.kw <= 0 || s.sh <= 0 || s.sw <= 0 || s.ph < 0 || s.pw < 0)
         return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: bad geometry", what);
+    if (s.g <= 0 || s.c % s.g != 0 || s.co % s.g != 0 || s.g > 65535)
+        return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: groups must divide the channel and filter counts", what);
     s.ho = (s.h + 2 * s.ph - s.kh) / s.sh + 1;             // (in + 2 pad - (k - 1) - 1) / stride + 1 (pam/pam_ops.py:137-138)
     s.wo = (s.w + 2 * s.pw - s.kw) / s.sw + 1;
     if (s.h + 2 * s.ph < s.kh || s.w + 2 * s.pw < s.kw) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: kernel larger than the padded image", what);
@@ -779,8 +789,8 @@ ConvSpace conv_space(const ConvShape& s, bool weight_gradient, bool has_off)
     w.tables = align256((size_t)(s.K() + s.L()) * sizeof(int2));
     size_t scaled_elems = !has_off ? 0 : weight_gradient ? (size_t)s.batch * s.co * s.L() : (size_t)s.co * s.K();
     w.scaled = align256(scaled_elems * sizeof(float));
-    size_t split = weight_gradient ? pam_hip_gemm_workspace_bytes(s.batch, s.co, s.K(), s.L())
-                                   : pam_hip_gemm_workspace_bytes(s.batch, s.co, s.L(), s.K());
+    size_t split = weight_gradient ? pam_hip_gemm_workspace_bytes(s.batch, s.cog(), s.K(), s.L())
+                                   : pam_hip_gemm_workspace_bytes(s.batch, s.cog(), s.L(), s.K());
     w.total = w.tables + w.scaled + split;
     return w;
 }
@@ -805,7 +815,7 @@ int input_gradient_shape(const char* what, const ConvShape& s, ConvShape& t)
 {
     if (s.sh != 1 || s.sw != 1) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: the input gradient in place needs stride 1", what);
     if (s.ph > s.kh - 1 || s.pw > s.kw - 1) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: padding larger than kernel - 1", what);
-    t = ConvShape{s.batch, s.co, s.ho, s.wo, s.c, s.kh, s.kw, 1, 1, s.kh - 1 - s.ph, s.kw - 1 - s.pw, 0, 0};
+    t = ConvShape{s.batch, s.co, s.ho, s.wo, s.c, s.kh, s.kw, 1, 1, s.kh - 1 - s.ph, s.kw - 1 - s.pw, 0, 0, s.g};
     int rc = conv_shape(what, t);
     if (rc != PAM_HIP_OK) return rc;
     if (t.ho != s.h || t.wo != s.w) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: geometry does not invert", what);
@@ -818,7 +828,7 @@ ConvSpace input_gradient_space(const ConvShape& t)
     ConvSpace w;
     w.tables = align256((size_t)(t.K() + t.L()) * sizeof(int2));
     w.scaled = align256((size_t)t.co * t.K() * sizeof(float));
-    w.total = w.tables + w.scaled + pam_hip_gemm_workspace_bytes(t.batch, t.co, t.L(), t.K());
+    w.total = w.tables + w.scaled + pam_hip_gemm_workspace_bytes(t.batch, t.cog(), t.L(), t.K());
     return w;
 }
 
@@ -902,9 +912,9 @@ int pam_hip_pam_bmm_bwd(PAM_HIP_MAT(l), PAM_HIP_MAT(r), PAM_HIP_MAT(mo), PAM_HIP
 }
 
 size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
-                                      long stride_h, long stride_w, long pad_h, long pad_w, int which, float offset)
+                                      long stride_h, long stride_w, long pad_h, long pad_w, long groups, int which, float offset)
 {
-    ConvShape s{batch, c, h, w, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    ConvShape s{batch, c, h, w, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0, groups};
     if (conv_shape("conv2d_workspace_bytes", s) != PAM_HIP_OK || batch == 0) return 0;
     if (which == 2) {
         ConvShape t;
@@ -915,10 +925,10 @@ size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long c
 }
 
 int pam_hip_conv2d_bwd_input(const float* dy, const float* w, const float* x, float* dx, long batch, long c, long h, long wd,
-                             long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                             long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w, long groups,
                              int exact, float offset, void* workspace, size_t workspace_bytes, void* stream)
 {
-    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0, groups};
     int rc = conv_shape("conv2d_bwd_input", s);
     if (rc != PAM_HIP_OK) return rc;
     ConvShape t;
@@ -932,24 +942,33 @@ int pam_hip_conv2d_bwd_input(const float* dy, const float* w, const float* x, fl
     rc = conv_prepare("conv2d_bwd_input", t, sp, workspace, workspace_bytes, st, cv, false);
     if (rc != PAM_HIP_OK) return rc;
     float* wf = (float*)((char*)workspace + sp.tables);
-    const long n = c * co * kh * kw;
+    const long n = c * s.cog() * kh * kw;
     // approximate: the offset goes into the flipped weights; exact: the product kernel applies it to its slope operand
-    hipLaunchKernelGGL(flip_weights_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w, wf, (int)c, (int)co, (int)kh, (int)kw,
-                       offset, (!exact && offset != 1.0f) ? 1 : 0);
-    const long K = t.K(), L = t.L();                  // K = co kh kw, L = h w
+    hipLaunchKernelGGL(flip_weights_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w, wf, (int)c, (int)s.cog(), (int)s.cg(),
+                       (int)kh, (int)kw, offset, (!exact && offset != 1.0f) ? 1 : 0);
+    const long K = t.K(), L = t.L();                  // K = (co / groups) kh kw, L = h w
     void* rest = (char*)workspace + sp.tables + sp.scaled; size_t rest_bytes = workspace_bytes - sp.tables - sp.scaled;
-    if (exact)        // dX[c, l] = sum_k pam_bwd(x[c, l], wf[c, k], dY patch[k, l]): x is the same for every term of an output
-        return gemm("conv2d_bwd_input", MODE_BWD_DR, batch, c, L, K, wf, 0, K, 1, dy, co * s.ho * s.wo, 0, 0, x, c * L, L, 1,
-                    dx, c * L, L, 1, offset, rest, rest_bytes, stream, &cv);
-    return gemm("conv2d_bwd_input", MODE_PAM, batch, c, L, K, wf, 0, K, 1, dy, co * s.ho * s.wo, 0, 0, nullptr, 0, 0, 0,
-                dx, c * L, L, 1, 1.0f, rest, rest_bytes, stream, &cv);
+    const long hw_out = s.ho * s.wo;
+    for (long gi = 0; gi < groups; ++gi) {            // one product per group: its filters' gradient slices in, its channels out
+        const float* wg = wf + gi * s.cg() * K;
+        const float* dyg = dy + gi * s.cog() * hw_out;
+        float* dxg = dx + gi * s.cg() * L;
+        if (exact)    // dX[c, l] = sum_k pam_bwd(x[c, l], wf[c, k], dY patch[k, l]): x is the same for every term of an output
+            rc = gemm("conv2d_bwd_input", MODE_BWD_DR, batch, s.cg(), L, K, wg, 0, K, 1, dyg, co * hw_out, 0, 0, x + gi * s.cg() * L, c * L, L, 1,
+                      dxg, c * L, L, 1, offset, rest, rest_bytes, stream, &cv);
+        else
+            rc = gemm("conv2d_bwd_input", MODE_PAM, batch, s.cg(), L, K, wg, 0, K, 1, dyg, co * hw_out, 0, 0, nullptr, 0, 0, 0,
+                      dxg, c * L, L, 1, 1.0f, rest, rest_bytes, stream, &cv);
+        if (rc != PAM_HIP_OK) return rc;
+    }
+    return PAM_HIP_OK;
 }
 
 int pam_hip_conv2d_fwd(const float* x, const float* w, float* y, long batch, long c, long h, long wd, long co, long kh, long kw,
-                       long stride_h, long stride_w, long pad_h, long pad_w, float offset,
+                       long stride_h, long stride_w, long pad_h, long pad_w, long groups, float offset,
                        void* workspace, size_t workspace_bytes, void* stream)
 {
-    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0, groups};
     int rc = conv_shape("conv2d_fwd", s);
     if (rc != PAM_HIP_OK) return rc;
     if (batch == 0) return PAM_HIP_OK;
@@ -970,16 +989,21 @@ int pam_hip_conv2d_fwd(const float* x, const float* w, float* y, long batch, lon
         wl = scaled;
     }
     const long K = s.K(), L = s.L();
-    // per image: Y[co, l] = sum_k W[co, k] (*) patches[k, l]
-    return gemm("conv2d_fwd", MODE_PAM, batch, co, L, K, wl, 0, K, 1, x, c * h * wd, 0, 0, nullptr, 0, 0, 0,
-                y, co * L, L, 1, 1.0f, (char*)workspace + sp.tables + sp.scaled, workspace_bytes - sp.tables - sp.scaled, stream, &cv);
+    // per image and group: Y[co, l] = sum_k W[co, k] (*) patches[k, l] over the group's channels
+    for (long gi = 0; gi < groups; ++gi) {
+        rc = gemm("conv2d_fwd", MODE_PAM, batch, s.cog(), L, K, wl + gi * s.cog() * K, 0, K, 1, x + gi * s.cg() * h * wd, c * h * wd, 0, 0,
+                  nullptr, 0, 0, 0, y + gi * s.cog() * L, co * L, L, 1, 1.0f,
+                  (char*)workspace + sp.tables + sp.scaled, workspace_bytes - sp.tables - sp.scaled, stream, &cv);
+        if (rc != PAM_HIP_OK) return rc;
+    }
+    return PAM_HIP_OK;
 }
 
 int pam_hip_conv2d_bwd_weight(const float* x, const float* dy, const float* w, float* dw, long batch, long c, long h, long wd,
-                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w,
+                              long co, long kh, long kw, long stride_h, long stride_w, long pad_h, long pad_w, long groups,
                               int exact, float offset, void* workspace, size_t workspace_bytes, void* stream)
 {
-    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0};
+    ConvShape s{batch, c, h, wd, co, kh, kw, stride_h, stride_w, pad_h, pad_w, 0, 0, groups};
     int rc = conv_shape("conv2d_bwd_weight", s);
     if (rc != PAM_HIP_OK) return rc;
     if (batch == 0) return PAM_HIP_OK;
@@ -992,9 +1016,6 @@ int pam_hip_conv2d_bwd_weight(const float* x, const float* dy, const float* w, f
     if (rc != PAM_HIP_OK) return rc;
     const long K = s.K(), L = s.L();
     void* rest = (char*)workspace + sp.tables + sp.scaled; size_t rest_bytes = workspace_bytes - sp.tables - sp.scaled;
-    if (exact)        // dW[co, k] = sum_l pam_bwd(W[co, k], patches[k, l], dY[co, l]); the offset goes with the patches
-        return gemm("conv2d_bwd_weight", MODE_BWD_DL, batch, co, K, L, dy, co * L, L, 1, x, c * h * wd, 0, 0, w, 0, K, 1,
-                    dw, co * K, K, 1, offset, rest, rest_bytes, stream, &cv);
     // approximate: dW[co, k] = sum_l patches[k, l] (*) (dY[co, l] (*) offset), the gradient scaled once up front
     const float* dl = dy;
     if (scale) {
@@ -1004,8 +1025,18 @@ int pam_hip_conv2d_bwd_weight(const float* x, const float* dy, const float* w, f
         hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, dy, scaled, n, offset);
         dl = scaled;
     }
-    return gemm("conv2d_bwd_weight", MODE_PAM, batch, co, K, L, dl, co * L, L, 1, x, c * h * wd, 0, 0, nullptr, 0, 0, 0,
-                dw, co * K, K, 1, 1.0f, rest, rest_bytes, stream, &cv);
+    for (long gi = 0; gi < groups; ++gi) {
+        const float* xg = x + gi * s.cg() * h * wd;
+        float* dwg = dw + gi * s.cog() * K;
+        if (exact)    // dW[co, k] = sum_l pam_bwd(W[co, k], patches[k, l], dY[co, l]); the offset goes with the patches
+            rc = gemm("conv2d_bwd_weight", MODE_BWD_DL, batch, s.cog(), K, L, dy + gi * s.cog() * L, co * L, L, 1, xg, c * h * wd, 0, 0,
+                      w + gi * s.cog() * K, 0, K, 1, dwg, co * K, K, 1, offset, rest, rest_bytes, stream, &cv);
+        else
+            rc = gemm("conv2d_bwd_weight", MODE_PAM, batch, s.cog(), K, L, dl + gi * s.cog() * L, co * L, L, 1, xg, c * h * wd, 0, 0,
+                      nullptr, 0, 0, 0, dwg, co * K, K, 1, 1.0f, rest, rest_bytes, stream, &cv);
+        if (rc != PAM_HIP_OK) return rc;
+    }
+    return PAM_HIP_OK;
 }
 
 }  // extern "C"

@@ -203,7 +203,7 @@ def input_gradient_in_place(W, stride, padding):
     return tuple(stride) == (1, 1) and padding[0] <= W.shape[2] - 1 and padding[1] <= W.shape[3] - 1
 
 
-def conv_in_place(X, W, dilation, approx_bwd, stride=(1, 1), padding=(0, 0)):
+def conv_in_place(X, W, dilation, approx_bwd, stride=(1, 1), padding=(0, 0), groups=1):
     """True when conv2d can run on the matrix kernel without unfolding X: fp32 GPU tensors,
     dilation 1, and, if the exact gradient with respect to X is wanted, a geometry for which that
     gradient is a convolution in place too (otherwise it needs the patches as a stored operand)."""
@@ -213,8 +213,11 @@ def conv_in_place(X, W, dilation, approx_bwd, stride=(1, 1), padding=(0, 0)):
         return False
     if dilation not in (1, (1, 1), [1, 1]):
         return False
+    wants_dx = torch.is_grad_enabled() and X.requires_grad
+    if groups != 1:          # grouped: the input gradient has no unfolded fallback here, it must be a convolution itself
+        return not wants_dx or input_gradient_in_place(W, stride, padding)
     approx_x, _ = _both(approx_bwd)
-    return approx_x or not (torch.is_grad_enabled() and X.requires_grad) or input_gradient_in_place(W, stride, padding)
+    return approx_x or not wants_dx or input_gradient_in_place(W, stride, padding)
 
 
 class conv2d_autograd(torch.autograd.Function):
@@ -223,12 +226,12 @@ class conv2d_autograd(torch.autograd.Function):
     into the weights, is applied to them before the product, so every term is the same."""
 
     @staticmethod
-    def forward(ctx, X, W, stride, padding, offset, approx_bwd):
-        ctx.stride, ctx.padding = stride, padding
+    def forward(ctx, X, W, stride, padding, offset, approx_bwd, groups=1):
+        ctx.stride, ctx.padding, ctx.groups = stride, padding, groups
         ctx.offset = _offset_value(offset)
         ctx.approx_bwd = approx_bwd
         ctx.save_for_backward(X, W)
-        return _abi.conv2d_fwd(X, W, stride, padding, ctx.offset)
+        return _abi.conv2d_fwd(X, W, stride, padding, ctx.offset, groups)
 
     @staticmethod
     def backward(ctx, dY):
@@ -238,13 +241,13 @@ class conv2d_autograd(torch.autograd.Function):
         dY = dY.contiguous()
         dX = dW = None
         if ctx.needs_input_grad[1]:
-            per_image = _abi.conv2d_bwd_weight(X, dY, W, ctx.stride, ctx.padding, not approx_w, off)
+            per_image = _abi.conv2d_bwd_weight(X, dY, W, ctx.stride, ctx.padding, not approx_w, off, ctx.groups)
             dW = per_image.sum(0).view(W.shape)
         if ctx.needs_input_grad[0] and input_gradient_in_place(W, ctx.stride, ctx.padding):
-            dX = _abi.conv2d_bwd_input(dY, W, X, ctx.padding, not approx_x, off)
+            dX = _abi.conv2d_bwd_input(dY, W, X, ctx.padding, not approx_x, off, ctx.groups)
         elif ctx.needs_input_grad[0]:
-            if not approx_x:
-                raise RuntimeError("exact gradient with respect to the convolution input needs the unfolded path")
+            if not approx_x or ctx.groups != 1:
+                raise RuntimeError("this gradient with respect to the convolution input needs the unfolded path")
             batch, co = dY.shape[:2]
             W2 = W.reshape(co, -1)
             if off != 1.0:
@@ -252,11 +255,11 @@ class conv2d_autograd(torch.autograd.Function):
             # gradient of the patch matrix, then the overlap-add that is unfold's gradient
             d_patches = k.pam_bmm_fwd(W2.t().unsqueeze(0).expand(batch, -1, -1), dY.view(batch, co, -1), False, True, 1.0)
             dX = torch.nn.functional.fold(d_patches, X.shape[2:], W.shape[2:], padding=ctx.padding, stride=ctx.stride)
-        return dX, dW, None, None, None, None
+        return dX, dW, None, None, None, None, None
 
 
-def conv2d(X, W, stride, padding, offset=None, approx_bwd=False):
-    return conv2d_autograd.apply(X, W, tuple(stride), tuple(padding), offset, approx_bwd)
+def conv2d(X, W, stride, padding, offset=None, approx_bwd=False, groups=1):
+    return conv2d_autograd.apply(X, W, tuple(stride), tuple(padding), offset, approx_bwd, groups)
 
 
 # ---------------------------------------------------------------- linear with the bias added in the product's epilogue

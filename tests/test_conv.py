@@ -114,9 +114,9 @@ def test_input_gradient_against_oracle(oracle, case, off):
 def test_input_gradient_rejects_other_strides():
     X = torch.randn(1, 2, 8, 8, device="cuda"); W = torch.randn(3, 2, 3, 3, device="cuda")
     lib = _abi.load_library()
-    assert lib.pam_hip_conv2d_workspace_bytes(1, 2, 8, 8, 3, 3, 3, 2, 2, 1, 1, 2, 1.0) == 0
+    assert lib.pam_hip_conv2d_workspace_bytes(1, 2, 8, 8, 3, 3, 3, 2, 2, 1, 1, 1, 2, 1.0) == 0
     dY = torch.randn(1, 3, 4, 4, device="cuda"); dX = torch.empty_like(X); ws = torch.empty(1 << 16, device="cuda")
-    rc = lib.pam_hip_conv2d_bwd_input(dY.data_ptr(), W.data_ptr(), X.data_ptr(), dX.data_ptr(), 1, 2, 8, 8, 3, 3, 3, 2, 2, 1, 1,
+    rc = lib.pam_hip_conv2d_bwd_input(dY.data_ptr(), W.data_ptr(), X.data_ptr(), dX.data_ptr(), 1, 2, 8, 8, 3, 3, 3, 2, 2, 1, 1, 1,
                                       0, 1.0, ws.data_ptr(), ws.numel() * 4, None)
     assert rc == -1 and b"stride 1" in lib.pam_hip_last_error()
     assert not pam_amd.fused.input_gradient_in_place(W, (2, 2), (1, 1)) and pam_amd.fused.input_gradient_in_place(W, (1, 1), (2, 2))
@@ -180,3 +180,83 @@ def _against_torch(X1, stride):
     Wt = conv.weight.detach().clone().requires_grad_()
     torch.nn.functional.conv2d(X2.detach(), Wt, None, padding=(1, 2), stride=stride).sum().backward()
     assert _close(conv.weight.grad, Wt.grad, 2e-6)
+
+
+GROUPED = [
+    # batch, c, h, w, co, kh, kw, stride, padding, groups
+    (2, 8, 9, 8, 12, 3, 3, (1, 1), (1, 1), 4),
+    (3, 6, 12, 10, 140, 3, 5, (2, 1), (0, 2), 2),        # 70 filters per group: more than one row tile
+    (2, 16, 7, 7, 16, 3, 3, (1, 1), (1, 1), 16),         # depthwise
+]
+
+
+@pytest.mark.parametrize("off", [None, OFF])
+@pytest.mark.parametrize("case", GROUPED)
+def test_grouped_convolution_against_oracle(oracle, case, off):
+    """pam.conv2d_group's arithmetic (pam/pam_ops.py:163-198) per group: forward, both weight gradients and, for
+    stride 1, both input gradients against the oracle's products on the unfolded slices."""
+    batch, c, h, w, co, kh, kw, stride, padding, G = case
+    cg, cog = c // G, co // G
+    rng = np.random.RandomState(11)
+    X = rng.standard_normal((batch, c, h, w)).astype(np.float32)
+    W = (rng.standard_normal((co, cg, kh, kw)) * 0.1).astype(np.float32)
+    X.reshape(-1)[rng.choice(X.size, 5, replace=False)] = [0.0, -0.0, 1e-40, -3e38, 7.0]
+    o = 1.0 if off is None else off
+    Xd, Wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
+    Y = _abi.conv2d_fwd(Xd, Wd, stride, padding, o, G)
+    ho, wo = Y.shape[2:]
+    L = ho * wo
+    dY = (rng.standard_normal((batch, co, ho, wo)) * 1e-2).astype(np.float32)
+    dYd = torch.from_numpy(dY).cuda()
+    dW_a = _abi.conv2d_bwd_weight(Xd, dYd, Wd, stride, padding, False, o, G).cpu().numpy()
+    dW_e = _abi.conv2d_bwd_weight(Xd, dYd, Wd, stride, padding, True, o, G).cpu().numpy()
+    stride_one = stride == (1, 1)
+    if stride_one:
+        dX_a = _abi.conv2d_bwd_input(dYd, Wd, Xd, padding, False, o, G).cpu().numpy()
+        dX_e = _abi.conv2d_bwd_input(dYd, Wd, Xd, padding, True, o, G).cpu().numpy()
+    for g in range(G):
+        Xg = np.ascontiguousarray(X[:, g * cg:(g + 1) * cg]); Wg = W[g * cog:(g + 1) * cog]; dYg = np.ascontiguousarray(dY[:, g * cog:(g + 1) * cog])
+        P = torch.nn.functional.unfold(torch.from_numpy(Xg), (kh, kw), padding=padding, stride=stride).numpy()        # [B, K, L]
+        K = P.shape[1]
+        W2 = Wg.reshape(cog, K)
+        Wl = W2 if off is None else oracle.pam(W2, np.float32(off))
+        want = oracle.gemm(np.broadcast_to(Wl, (batch, cog, K)), P, kchunk=_plan(batch, cog, L, K))
+        assert_same_bits(Y[:, g * cog:(g + 1) * cog].cpu().numpy().reshape(batch, cog, L), want, f"grouped forward, group {g}")
+        Pt = np.ascontiguousarray(P.transpose(0, 2, 1)); d2 = dYg.reshape(batch, cog, L); plan = _plan(batch, cog, K, L)
+        dl = d2 if off is None else oracle.pam(d2, np.float32(off))
+        assert_same_bits(dW_a[:, g * cog:(g + 1) * cog], oracle.gemm(dl, Pt, kchunk=plan), f"grouped weight gradient, group {g}")
+        want = oracle.gemm(d2, Pt, mode=oracle.MODE_BWD_DELTA_L, D=np.broadcast_to(W2, (batch, cog, K)), offset=off, kchunk=plan)
+        assert_same_bits(dW_e[:, g * cog:(g + 1) * cog], want, f"grouped exact weight gradient, group {g}")
+        if stride_one:
+            Pd = torch.nn.functional.unfold(torch.from_numpy(dYg), (kh, kw), padding=(kh - 1 - padding[0], kw - 1 - padding[1])).numpy()
+            Kt = Pd.shape[1]
+            Wf = np.ascontiguousarray(Wg.transpose(1, 0, 2, 3)[:, :, ::-1, ::-1]).reshape(cg, Kt)
+            plan = _plan(batch, cg, h * w, Kt)
+            Wfl = Wf if off is None else oracle.pam(Wf, np.float32(off))
+            assert_same_bits(dX_a[:, g * cg:(g + 1) * cg].reshape(batch, cg, h * w), oracle.gemm(np.broadcast_to(Wfl, (batch, cg, Kt)), Pd, kchunk=plan),
+                             f"grouped input gradient, group {g}")
+            want = oracle.gemm(np.broadcast_to(Wf, (batch, cg, Kt)), Pd, mode=oracle.MODE_BWD_DELTA_R, D=Xg.reshape(batch, cg, h * w), offset=off, kchunk=plan)
+            assert_same_bits(dX_e[:, g * cg:(g + 1) * cg].reshape(batch, cg, h * w), want, f"grouped exact input gradient, group {g}")
+
+
+@pytest.mark.parametrize("stride", [(1, 1), (2, 2)])
+@pytest.mark.parametrize("approx", [True, False])
+def test_grouped_module_matches_unfolded_composition(approx, stride):
+    """pam.Conv2d with groups: patches in place against unfold + bmm on the same GPU, values and gradients."""
+    torch.manual_seed(3)
+    X = torch.randn(3, 8, 10, 9, device="cuda"); g = None
+    res = {}
+    for implicit in (True, False):
+        composites.implicit_conv = implicit
+        try:
+            torch.manual_seed(4)
+            conv = pam_amd.Conv2d(8, 12, 3, padding=1, stride=stride, groups=4, approx_bwd=approx, offset=OFF).cuda()
+            Xr = X.clone().requires_grad_()
+            Y = conv(Xr)
+            g = torch.randn_like(Y) if g is None else g
+            Y.backward(g)
+            res[implicit] = (Y.detach(), Xr.grad, conv.weight.grad, conv.bias.grad)
+        finally:
+            composites.implicit_conv = True
+    for a, c in zip(res[True], res[False]):
+        assert a.shape == c.shape and _close(a, c)
