@@ -205,6 +205,60 @@ __device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)
     return total;
 }
 
+// Rows too long for registers are swept in blocks of 64 x kBlock values, a lane meeting its elements in the
+// same ascending order as in the register variants (so the row sums are the same sums); the later sweeps find
+// the row in cache.  The same two-step scheme applies: branch-free forms first, the checked ones if any value
+// left the normal range.
+constexpr int kBlock = 8;
+
+template <class F>
+__device__ __forceinline__ void for_blocks(const float* __restrict__ row, long n, int lane, float fill, F&& body)
+{
+    for (long base = 0; base < n; base += 64L * kBlock) {
+        float v[kBlock];
+#pragma unroll
+        for (int c = 0; c < kBlock; ++c) { const long i = base + lane + 64L * c; v[c] = i < n ? row[i] : fill; }
+#pragma unroll
+        for (int c = 0; c < kBlock; ++c) { const long i = base + lane + 64L * c; body(i, i < n, v[c]); }
+    }
+}
+
+// the same over two rows at once (all loads of a block are issued before its arithmetic)
+template <class F>
+__device__ __forceinline__ void for_blocks2(const float* __restrict__ row_a, const float* __restrict__ row_b, long n, int lane,
+                                            float fill_a, float fill_b, F&& body)
+{
+    for (long base = 0; base < n; base += 64L * kBlock) {
+        float a[kBlock], b[kBlock];
+#pragma unroll
+        for (int c = 0; c < kBlock; ++c) {
+            const long i = base + lane + 64L * c;
+            a[c] = i < n ? row_a[i] : fill_a; b[c] = i < n ? row_b[i] : fill_b;
+        }
+#pragma unroll
+        for (int c = 0; c < kBlock; ++c) { const long i = base + lane + 64L * c; body(i, i < n, a[c], b[c]); }
+    }
+}
+
+template <class M>
+__device__ __forceinline__ float softmax_stream(const float* __restrict__ xr, float* __restrict__ yr, long n, int lane, float shift, M& m)
+{
+    auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
+    float p = 0.0f;
+    for_blocks(xr, n, lane, kNegInf, [&](long, bool, float x) {
+        const bool masked = f2u(x) == 0xff800000u;
+        const float e = weight(x, masked);
+        p = p + (masked ? 0.0f : e);
+    });
+    const float total = wave_sum(p);
+    for_blocks(xr, n, lane, kNegInf, [&](long i, bool inside, float x) {
+        const bool masked = f2u(x) == 0xff800000u;
+        const float q = m.div(masked ? 1.0f : weight(x, masked), total);
+        if (inside) yr[i] = masked ? m.zero_over(total) : q;
+    });
+    return total;
+}
+
 template <int CH>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC(CH)))) void softmax_fwd_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                               float* __restrict__ row_sum, float* __restrict__ shift_out,
@@ -227,8 +281,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
-            total = wave_sum(stream_sum(xr, n, lane, [&](long, float v) { return softmax_weight(v, shift, o); }));
-            for (long i = lane; i < n; i += 64) yr[i] = pad_div_off(softmax_weight(xr[i], shift, o), total, o.off, o.has);
+            Unchecked u{o};
+            total = softmax_stream(xr, yr, n, lane, shift, u);
+            if (!wave_valid(u)) { Checked k{o}; total = softmax_stream(xr, yr, n, lane, shift, k); }
         }
         if (lane == 0) row_sum[r] = total;
     }
@@ -330,11 +385,36 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) dr[i] = out[c]; }
         } else {
-            const float dtotal = wave_sum(stream_sum(xr, n, lane, [&](long i, float v) {
-                return softmax_dsum_term(softmax_weight(v, shift, o), total, gr[i], o, ap); }));
-            for (long i = lane; i < n; i += 64) {
-                const float v = xr[i];
-                dr[i] = softmax_dx(v, softmax_weight(v, shift, o), gr[i], inv, dtotal, shift, o, ap);
+            bool done = false;
+            if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient, branch-free forms first
+                Unchecked m{o};
+                const float inv_u = m.div(1.0f, total);
+                auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
+                float p = 0.0f;
+                for_blocks2(xr, gr, n, lane, kNegInf, 1.0f, [&](long, bool inside, float x, float gi) {
+                    const bool masked = f2u(x) == 0xff800000u;
+                    const float e = weight(x, masked);
+                    const float term = -m.mul(m.div(m.div(e, total), total), masked ? 1.0f : gi);
+                    if (masked && inside) m.sp.see(f2u(gi) & ~kSign);         // -(0 (*) g) is a zero only for finite g
+                    if (inside && !masked) p = p + term;
+                });
+                const float dtotal = wave_sum(p);
+                for_blocks2(xr, gr, n, lane, kNegInf, 1.0f, [&](long i, bool inside, float x, float gi) {
+                    const bool masked = f2u(x) == 0xff800000u;
+                    const float e = weight(x, masked);
+                    const float de = m.mul(inv_u, masked ? 1.0f : gi) + dtotal;
+                    const float d = m.mul(m.mul(m.mul(e, kLn2), de), kLog2E);
+                    if (inside) dr[i] = masked ? 0.0f : d;
+                });
+                done = wave_valid(m);
+            }
+            if (!done) {
+                const float dtotal = wave_sum(stream_sum(xr, n, lane, [&](long i, float v) {
+                    return softmax_dsum_term(softmax_weight(v, shift, o), total, gr[i], o, ap); }));
+                for (long i = lane; i < n; i += 64) {
+                    const float v = xr[i];
+                    dr[i] = softmax_dx(v, softmax_weight(v, shift, o), gr[i], inv, dtotal, shift, o, ap);
+                }
             }
         }
     }
@@ -366,7 +446,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
-        auto weight = [&](long, float v) { return exp2_op(scaled(v, o, false) - shift, o); };
         if constexpr (CH > 0) {
             float xv[CH];
             load_row<CH>(xv, xr, n, lane, 0.0f);
@@ -379,9 +458,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) y[r * n + i] = xv[c] - out; }
             }
         } else {
-            const float out = pad_div_off(shift + log2_op(wave_sum(stream_sum(xr, n, lane, weight)), o), kLog2E, o.off, o.has);
+            auto sweep = [&](auto& m) {
+                float p = 0.0f;
+                for_blocks(xr, n, lane, 0.0f, [&](long, bool inside, float v) {
+                    const float e = m.exp2(inside ? m.mul(v, kLog2E) - shift : 0.5f);
+                    if (inside) p = p + e;
+                });
+                return m.div(shift + m.log2(wave_sum(p)), kLog2E);
+            };
+            Unchecked u{o};
+            float out = sweep(u);
+            if (!wave_valid(u)) { Checked k{o}; out = sweep(k); }
             if (lse && lane == 0) lse[r] = out;
-            if (y) for (long i = lane; i < n; i += 64) y[r * n + i] = xr[i] - out;
+            if (y) for_blocks(xr, n, lane, 0.0f, [&](long i, bool inside, float v) { if (inside) y[r * n + i] = v - out; });
         }
     }
 }
@@ -457,11 +546,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
-            const float mu = pad_div_off(wave_sum(stream_sum(xr, n, lane, [](long, float v) { return v; })), count, o.off, o.has);
-            const float var = pad_div_off(wave_sum(stream_sum(xr, n, lane, [&](long, float v) {
-                float c = v - mu; return pam_mul_off(c, c, o.off, o.has); })), count, o.off, o.has);
-            const float denom = root_op(var + eps, o);
-            for (long i = lane; i < n; i += 64) yr[i] = layer_norm_out(xr[i] - mu, denom, i, weight, bias, o);
+            auto sweep = [&](auto& m) {
+                float p = 0.0f;
+                for_blocks(xr, n, lane, 0.0f, [&](long, bool, float v) { p = p + v; });            // the fill adds +0
+                const float mu = m.div(wave_sum(p), count);
+                p = 0.0f;
+                for_blocks(xr, n, lane, 0.0f, [&](long, bool inside, float v) {
+                    const float c = v - mu, sq = m.mul(c, c);                                    // past the end: -mu, a stand-in
+                    if (inside) p = p + sq;
+                });
+                const float denom = m.root(m.div(wave_sum(p), count) + eps);
+                for_blocks(xr, n, lane, 0.0f, [&](long i, bool inside, float v) {
+                    float r = m.div(v - mu, denom);
+                    if (weight) r = m.mul(r, inside ? weight[i] : 1.0f);
+                    if (bias) r = r + (inside ? bias[i] : 0.0f);
+                    if (inside) yr[i] = r;
+                });
+            };
+            Unchecked u{o};
+            sweep(u);
+            if (!wave_valid(u)) { Checked k{o}; sweep(k); }
         }
     }
 }
