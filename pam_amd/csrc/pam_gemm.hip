@@ -677,7 +677,8 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
 {
     if (batch < 0 || M < 0 || N < 0 || K < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: negative size", what);
     if (batch == 0 || M == 0 || N == 0) return PAM_HIP_OK;
-    if (!l || !r || !y || (mode >= MODE_BWD_DL && !d)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: null pointer", what);
+    // with K == 0 the operands are empty (and may be null): the sums over nothing are +0 (plus the bias)
+    if (((!l || !r) && K > 0) || !y || (mode >= MODE_BWD_DL && !d)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: null pointer", what);
     if (M > (1L << 30) || N > (1L << 30) || K > (1L << 30) || batch > 65535 || ((M + 63) / 64) * ((N + 63) / 64) > 0x7fffffffL)
         return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: dimension too large (sizes <= 2^30, batch <= 65535, output tiles < 2^31)", what);
     hipStream_t st = (hipStream_t)stream;

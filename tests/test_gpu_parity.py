@@ -550,3 +550,27 @@ def test_both_gradients_in_one_pass(K, oracle, off):
                 cuda_bindings.paired_gradients = True
         assert_same_bits(res[True][0], res[False][0], "dA paired against single")
         assert_same_bits(res[True][1], res[False][1], "dB paired against single")
+
+
+def test_degenerate_shapes(K, oracle):
+    """Empty operands and a zero-length inner dimension: no launch faults, outputs of the right shape, and a
+    sum over nothing is +0 (the accumulators start there); empty rows for the row-wise kernels."""
+    import pam_amd
+    from pam_amd import _abi
+    z = lambda *s: torch.zeros(*s, device="cuda")
+    assert K.pam_matmul_fwd(z(0, 8), z(8, 5), True, True, 1.0).shape == (0, 5)
+    assert K.pam_matmul_fwd(z(7, 8), z(8, 0), True, True, 1.0).shape == (7, 0)
+    y = K.pam_matmul_fwd(torch.full((7, 0), 3.0, device="cuda"), z(0, 5), True, True, 1.0)
+    assert y.shape == (7, 5) and (host(y).view(np.uint32) == 0).all()
+    y = K.pam_bmm_fwd(z(3, 4, 0), z(3, 0, 6), True, True, 1.0)
+    assert y.shape == (3, 4, 6) and (host(y).view(np.uint32) == 0).all()
+    assert K.pam_bmm_fwd(z(0, 4, 5), z(0, 5, 6), True, True, 1.0).shape == (0, 4, 6)
+    assert K.pam_matmul_bwd(z(7, 0), z(0, 5), z(7, 5), True, True, True, 1.0).shape == (7, 5)
+    R = _abi.HipRowKernels()
+    ys, rs, sh = R.softmax_fwd(z(0, 16), 1.0)
+    assert ys.shape == (0, 16) and rs.shape == (0,)
+    assert R.row_mean_fwd(z(0, 16), 1.0).shape == (0,)
+    with pytest.raises(RuntimeError):                    # as in the reference: the global maximum of nothing (pam/pam_ops.py:318)
+        pam_amd.softmax(z(4, 0), dim=-1)
+    assert _abi.conv2d_fwd(z(0, 3, 8, 8), z(4, 3, 3, 3), (1, 1), (1, 1), 1.0).shape == (0, 4, 8, 8)
+    assert K.pam_fwd(z(0), z(0), 1.0).shape == (0,)
