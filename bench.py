@@ -92,6 +92,12 @@ def main():
         for fn in products.values():
             fn()
 
+    # Clocks and the launch queue need some tens of milliseconds of work to settle; the same products run for a
+    # moment before the W warm-up steps so that a short timed run (small K) measures the settled rate too.
+    ramp_end = time.perf_counter() + 0.25
+    while time.perf_counter() < ramp_end:
+        step()
+    torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
