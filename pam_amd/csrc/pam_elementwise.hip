@@ -137,7 +137,7 @@ __global__ __launch_bounds__(kThreads) void ew_vec_kernel(const v4f* __restrict_
         for (int u = 0; u < kUnroll; ++u) {
             size_t i = base + (size_t)u * kThreads;
             if (i < nvec) {
-                v4f r;
+                v4f r = {};
                 bool done = false;
                 if constexpr (HasFast<Op>::value) {
                     if (op.has_fast()) {

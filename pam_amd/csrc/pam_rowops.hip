@@ -70,8 +70,6 @@ __device__ __forceinline__ float scaled(float x, Offset o, bool mask_inf)
 
 // exp2 through the kernel entry point of that name: pa_exp2(t (*) log2(2)) (pam/cuda_bindings.py:246)
 __device__ __forceinline__ float exp2_op(float t, Offset o) { return exp2_entry(t, o.off, o.has); }
-// log2 likewise: pa_log2(v) (/) log2(2)
-__device__ __forceinline__ float log2_op(float v, Offset o) { return log2_entry(v, o.off, o.has); }
 
 // ---------------------------------------------------------------- global maximum of the scaled input
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -275,13 +273,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if constexpr (CH > 0) {
             float xv[CH], out[CH];
             load_row<CH>(xv, xr, n, lane, kNegInf);            // the fill has weight zero
-            Unchecked u{o};
+            Unchecked u{o, Span()};
             total = softmax_row<CH>(xv, out, shift, u);
             if (!wave_valid(u)) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k); }
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
-            Unchecked u{o};
+            Unchecked u{o, Span()};
             total = softmax_stream(xr, yr, n, lane, shift, u);
             if (!wave_valid(u)) { Checked k{o}; total = softmax_stream(xr, yr, n, lane, shift, k); }
         }
@@ -366,7 +364,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             load_row<CH>(g, gr, n, lane, 0.0f);
             bool done = false;
             if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient has an unchecked form
-                Unchecked u{o};
+                Unchecked u{o, Span()};
                 softmax_grad_row_approx<CH>(xv, g, out, total, shift, lane, n, u);
                 done = wave_valid(u);
             }
@@ -387,7 +385,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         } else {
             bool done = false;
             if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient, branch-free forms first
-                Unchecked m{o};
+                Unchecked m{o, Span()};
                 const float inv_u = m.div(1.0f, total);
                 auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
                 float p = 0.0f;
@@ -449,7 +447,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if constexpr (CH > 0) {
             float xv[CH];
             load_row<CH>(xv, xr, n, lane, 0.0f);
-            Unchecked u{o};
+            Unchecked u{o, Span()};
             float out = logsumexp_row<CH>(xv, shift, lane, n, u);
             if (!wave_valid(u)) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lane, n, k); }
             if (lse && lane == 0) lse[r] = out;
@@ -466,7 +464,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 });
                 return m.div(shift + m.log2(wave_sum(p)), kLog2E);
             };
-            Unchecked u{o};
+            Unchecked u{o, Span()};
             float out = sweep(u);
             if (!wave_valid(u)) { Checked k{o}; out = sweep(k); }
             if (lse && lane == 0) lse[r] = out;
@@ -489,18 +487,6 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restr
 }
 
 // ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
-// pow(v, 0.5) = exp2(log2(v) (*) 0.5), zero at zero (pam/pam_ops.py:70-79)
-__device__ __forceinline__ float root_op(float v, Offset o) { return pow_half(v, o.off, o.has); }
-
-__device__ __forceinline__ float layer_norm_out(float centred, float denom, long i, const float* __restrict__ weight,
-                                               const float* __restrict__ bias, Offset o)
-{
-    float out = pad_div_off(centred, denom, o.off, o.has);
-    if (weight) out = pam_mul_off(out, weight[i], o.off, o.has);
-    if (bias) out = out + bias[i];
-    return out;
-}
-
 template <int CH, class M>
 __device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&out)[CH], const float* __restrict__ weight,
                                                const float* __restrict__ bias, int lane, long n, float count, float eps, M& m)
@@ -540,7 +526,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if constexpr (CH > 0) {
             float xv[CH], out[CH];
             load_row<CH>(xv, xr, n, lane, 0.0f);
-            Unchecked u{o};
+            Unchecked u{o, Span()};
             layer_norm_row<CH>(xv, out, weight, bias, lane, n, count, eps, u);
             if (!wave_valid(u)) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lane, n, count, eps, k); }
 #pragma unroll
@@ -563,7 +549,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                     if (inside) yr[i] = r;
                 });
             };
-            Unchecked u{o};
+            Unchecked u{o, Span()};
             sweep(u);
             if (!wave_valid(u)) { Checked k{o}; sweep(k); }
         }
@@ -659,7 +645,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
         if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o};
+            GradUnchecked u{o, Span()};
             logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lane, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -729,7 +715,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
         if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o};
+            GradUnchecked u{o, Span()};
             logsumexp_grad_stream(x + r * n, gr, dx + r * n, g_row, log_softmax != 0, shift, lane, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -863,7 +849,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         float* tr = (weight && dw_terms) ? dw_terms + r * n : nullptr;
         bool done = false;
         if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o};
+            GradUnchecked u{o, Span()};
             layer_norm_grad_stream(x + r * n, gy + r * n, weight, dx + r * n, tr, lane, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -886,7 +872,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >
         if (ap.a && ap.b && ap.e) {
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
-            GradUnchecked u{o};
+            GradUnchecked u{o, Span()};
             layer_norm_grad_row<CH>(cen, g, terms, weight, lane, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
