@@ -210,31 +210,31 @@ __device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)
 constexpr int kBlock = 8;
 
 template <class F>
-__device__ __forceinline__ void for_blocks(const float* __restrict__ row, long n, int lane, float fill, F&& body)
+__device__ __forceinline__ void for_blocks(const float* __restrict__ row, int n, int lane, float fill, F&& body)
 {
-    for (long base = 0; base < n; base += 64L * kBlock) {
+    for (int base = 0; base < n; base += 64 * kBlock) {
         float v[kBlock];
 #pragma unroll
-        for (int c = 0; c < kBlock; ++c) { const long i = base + lane + 64L * c; v[c] = i < n ? row[i] : fill; }
+        for (int c = 0; c < kBlock; ++c) { const int i = base + lane + 64 * c; v[c] = i < n ? row[i] : fill; }
 #pragma unroll
-        for (int c = 0; c < kBlock; ++c) { const long i = base + lane + 64L * c; body(i, i < n, v[c]); }
+        for (int c = 0; c < kBlock; ++c) { const int i = base + lane + 64 * c; body(i, i < n, v[c]); }
     }
 }
 
 // the same over two rows at once (all loads of a block are issued before its arithmetic)
 template <class F>
-__device__ __forceinline__ void for_blocks2(const float* __restrict__ row_a, const float* __restrict__ row_b, long n, int lane,
+__device__ __forceinline__ void for_blocks2(const float* __restrict__ row_a, const float* __restrict__ row_b, int n, int lane,
                                             float fill_a, float fill_b, F&& body)
 {
-    for (long base = 0; base < n; base += 64L * kBlock) {
+    for (int base = 0; base < n; base += 64 * kBlock) {
         float a[kBlock], b[kBlock];
 #pragma unroll
         for (int c = 0; c < kBlock; ++c) {
-            const long i = base + lane + 64L * c;
+            const int i = base + lane + 64 * c;
             a[c] = i < n ? row_a[i] : fill_a; b[c] = i < n ? row_b[i] : fill_b;
         }
 #pragma unroll
-        for (int c = 0; c < kBlock; ++c) { const long i = base + lane + 64L * c; body(i, i < n, a[c], b[c]); }
+        for (int c = 0; c < kBlock; ++c) { const int i = base + lane + 64 * c; body(i, i < n, a[c], b[c]); }
     }
 }
 
@@ -243,13 +243,13 @@ __device__ __forceinline__ float softmax_stream(const float* __restrict__ xr, fl
 {
     auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
     float p = 0.0f;
-    for_blocks(xr, n, lane, kNegInf, [&](long, bool, float x) {
+    for_blocks(xr, (int)n, lane, kNegInf, [&](long, bool, float x) {
         const bool masked = f2u(x) == 0xff800000u;
         const float e = weight(x, masked);
         p = p + (masked ? 0.0f : e);
     });
     const float total = wave_sum(p);
-    for_blocks(xr, n, lane, kNegInf, [&](long i, bool inside, float x) {
+    for_blocks(xr, (int)n, lane, kNegInf, [&](long i, bool inside, float x) {
         const bool masked = f2u(x) == 0xff800000u;
         const float q = m.div(masked ? 1.0f : weight(x, masked), total);
         if (inside) yr[i] = masked ? m.zero_over(total) : q;
@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 const float inv_u = m.div(1.0f, total);
                 auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
                 float p = 0.0f;
-                for_blocks2(xr, gr, n, lane, kNegInf, 1.0f, [&](long, bool inside, float x, float gi) {
+                for_blocks2(xr, gr, (int)n, lane, kNegInf, 1.0f, [&](long, bool inside, float x, float gi) {
                     const bool masked = f2u(x) == 0xff800000u;
                     const float e = weight(x, masked);
                     const float term = -m.mul(m.div(m.div(e, total), total), masked ? 1.0f : gi);
@@ -397,7 +397,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                     if (inside && !masked) p = p + term;
                 });
                 const float dtotal = wave_sum(p);
-                for_blocks2(xr, gr, n, lane, kNegInf, 1.0f, [&](long i, bool inside, float x, float gi) {
+                for_blocks2(xr, gr, (int)n, lane, kNegInf, 1.0f, [&](long i, bool inside, float x, float gi) {
                     const bool masked = f2u(x) == 0xff800000u;
                     const float e = weight(x, masked);
                     const float de = m.mul(inv_u, masked ? 1.0f : gi) + dtotal;
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         } else {
             auto sweep = [&](auto& m) {
                 float p = 0.0f;
-                for_blocks(xr, n, lane, 0.0f, [&](long, bool inside, float v) {
+                for_blocks(xr, (int)n, lane, 0.0f, [&](long, bool inside, float v) {
                     const float e = m.exp2(inside ? m.mul(v, kLog2E) - shift : 0.5f);
                     if (inside) p = p + e;
                 });
@@ -468,7 +468,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             float out = sweep(u);
             if (!wave_valid(u)) { Checked k{o}; out = sweep(k); }
             if (lse && lane == 0) lse[r] = out;
-            if (y) for_blocks(xr, n, lane, 0.0f, [&](long i, bool inside, float v) { if (inside) y[r * n + i] = v - out; });
+            if (y) for_blocks(xr, (int)n, lane, 0.0f, [&](long i, bool inside, float v) { if (inside) y[r * n + i] = v - out; });
         }
     }
 }
@@ -534,15 +534,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         } else {
             auto sweep = [&](auto& m) {
                 float p = 0.0f;
-                for_blocks(xr, n, lane, 0.0f, [&](long, bool, float v) { p = p + v; });            // the fill adds +0
+                for_blocks(xr, (int)n, lane, 0.0f, [&](long, bool, float v) { p = p + v; });            // the fill adds +0
                 const float mu = m.div(wave_sum(p), count);
                 p = 0.0f;
-                for_blocks(xr, n, lane, 0.0f, [&](long, bool inside, float v) {
+                for_blocks(xr, (int)n, lane, 0.0f, [&](long, bool inside, float v) {
                     const float c = v - mu, sq = m.mul(c, c);                                    // past the end: -mu, a stand-in
                     if (inside) p = p + sq;
                 });
                 const float denom = m.root(m.div(wave_sum(p), count) + eps);
-                for_blocks(xr, n, lane, 0.0f, [&](long i, bool inside, float v) {
+                for_blocks(xr, (int)n, lane, 0.0f, [&](long i, bool inside, float v) {
                     float r = m.div(v - mu, denom);
                     if (weight) r = m.mul(r, inside ? weight[i] : 1.0f);
                     if (bias) r = r + (inside ? bias[i] : 0.0f);
@@ -660,21 +660,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 // order as in the register variant, so the sums are the same sums.
 template <class G>
 __device__ __forceinline__ void logsumexp_grad_stream(const float* __restrict__ xr, const float* __restrict__ gr, float* __restrict__ dr,
-                                                      float g_row, bool log_softmax, float shift, int lane, long n, G& m)
+                                                      float g_row, bool log_softmax, float shift, int lane, long rowlen, G& m)
 {
+    const int n = (int)rowlen;                    // at most 2^30: 32-bit index arithmetic
     constexpr int U = 8;
     float p = 0.0f, q = 0.0f;
-    for (long base = 0; base < n; base += 64L * U) {
+    for (int base = 0; base < n; base += 64 * U) {
         float xv[U], gy[U];
 #pragma unroll
         for (int c = 0; c < U; ++c) {
-            const long i = base + lane + 64L * c; const bool inside = i < n;
+            const int i = base + lane + 64 * c; const bool inside = i < n;
             xv[c] = inside ? xr[i] : 1.0f;
             gy[c] = (inside && log_softmax) ? gr[i] : 0.0f;
         }
 #pragma unroll
         for (int c = 0; c < U; ++c) {
-            const bool inside = base + lane + 64L * c < n;
+            const bool inside = base + lane + 64 * c < n;
             const float sc = m.mul(xv[c], kLog2E) - shift;
             const float e = m.exp2(inside ? sc : 0.5f);
             if (inside) { p = p + e; q = q + gy[c]; }
@@ -685,17 +686,17 @@ __device__ __forceinline__ void logsumexp_grad_stream(const float* __restrict__ 
     const float u = shift + m.log2(total);
     const float du = m.div_da(u, kLog2E, g_out);
     const float dtotal = m.log2_dx(total, du);
-    for (long base = 0; base < n; base += 64L * U) {
+    for (int base = 0; base < n; base += 64 * U) {
         float xv[U], gy[U];
 #pragma unroll
         for (int c = 0; c < U; ++c) {
-            const long i = base + lane + 64L * c; const bool inside = i < n;
+            const int i = base + lane + 64 * c; const bool inside = i < n;
             xv[c] = inside ? xr[i] : 1.0f;
             gy[c] = (inside && log_softmax) ? gr[i] : 0.0f;
         }
 #pragma unroll
         for (int c = 0; c < U; ++c) {
-            const long i = base + lane + 64L * c; const bool inside = i < n;
+            const int i = base + lane + 64 * c; const bool inside = i < n;
             const float sc = m.mul(xv[c], kLog2E) - shift;
             const float d = m.mul_da(xv[c], kLog2E, m.exp2_dx(inside ? sc : 0.5f, dtotal));
             if (inside) dr[i] = log_softmax ? gy[c] + d : d;
@@ -785,16 +786,17 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
 template <class G>
 __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__ xr, const float* __restrict__ gr,
                                                        const float* __restrict__ weight, float* __restrict__ dr,
-                                                       float* __restrict__ tr, int lane, long n, float count, float eps, G& m)
+                                                       float* __restrict__ tr, int lane, long rowlen, float count, float eps, G& m)
 {
+    const int n = (int)rowlen;                    // at most 2^30: 32-bit index arithmetic
     float p = 0.0f;
 #pragma unroll 4
-    for (long i = lane; i < n; i += 64) p = p + xr[i];
+    for (int i = lane; i < n; i += 64) p = p + xr[i];
     const float s1 = wave_sum(p);
     const float mu = m.div(s1, count);
     p = 0.0f;
 #pragma unroll 4
-    for (long i = lane; i < n; i += 64) { const float c = xr[i] - mu; p = p + m.mul(c, c); }
+    for (int i = lane; i < n; i += 64) { const float c = xr[i] - mu; p = p + m.mul(c, c); }
     const float s2 = wave_sum(p);
     const float v = m.div(s2, count) + eps;
     const float lg = m.log2(v);
@@ -802,7 +804,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
     const float root = m.exp2(half);
     const float denom = v == 0.0f ? 0.0f : root;
     // the upstream gradient behind the weight product (and that product's term for the weight gradient)
-    auto behind_weight = [&](long i, float c, bool store_term) {
+    auto behind_weight = [&](int i, float c, bool store_term) {
         float g = gr[i];
         if (weight) {
             const float xn = m.div(c, denom), wi = weight[i];
@@ -813,7 +815,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
     };
     p = 0.0f;
 #pragma unroll 4
-    for (long i = lane; i < n; i += 64) {
+    for (int i = lane; i < n; i += 64) {
         const float c = xr[i] - mu;
         p = p + m.div_db(c, denom, behind_weight(i, c, true));
     }
@@ -825,7 +827,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
     const float ds2 = m.div_da(s2, count, d);
     p = 0.0f;
 #pragma unroll 4
-    for (long i = lane; i < n; i += 64) {
+    for (int i = lane; i < n; i += 64) {
         const float c = xr[i] - mu;
         float dc = m.div_da(c, denom, behind_weight(i, c, false));
         dc = dc + m.mul_da(c, c, ds2);
@@ -835,7 +837,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
     }
     const float ds1 = m.div_da(s1, count, -wave_sum(p));
 #pragma unroll 4
-    for (long i = lane; i < n; i += 64) dr[i] = dr[i] + ds1;
+    for (int i = lane; i < n; i += 64) dr[i] = dr[i] + ds1;
 }
 
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void layer_norm_bwd_stream_kernel(
