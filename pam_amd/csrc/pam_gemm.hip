@@ -72,6 +72,7 @@ struct GemmArgs {
     const float* bias;           // one value per output column, added once after the sum, or null
     int M, N, K;
     int ksplit, kchunk;          // kchunk is a multiple of 32; ksplit == 1 means no split
+    int xcd_chunk, tiles;        // xcd_chunk > 0: work-group x takes tile (x % 8) * xcd_chunk + x / 8 (see the launch)
     float off; int has_off;
 };
 
@@ -290,8 +291,13 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     const int tid = threadIdx.x, tx = tid % TXN, ty = tid / TXN;
     const int wave = tid / 64, lane = tid % 64;
     const int zb = blockIdx.z, zs = blockIdx.y;
-    const int ntn = (g.N + BN - 1) / BN;                  // consecutive work-groups share L rows
-    const int row0 = (blockIdx.x / ntn) * BM, col0 = (blockIdx.x % ntn) * BN;
+    const int ntn = (g.N + BN - 1) / BN;                  // consecutive tiles share L rows
+    int tile = blockIdx.x;
+    if (g.xcd_chunk > 0) {                                // one contiguous range of tiles per XCD (its own L2)
+        tile = (int)(blockIdx.x % 8) * g.xcd_chunk + (int)(blockIdx.x / 8);
+        if (tile >= g.tiles) return;                      // the ranges are rounded up: a few work-groups have nothing to do
+    }
+    const int row0 = (tile / ntn) * BM, col0 = (tile % ntn) * BN;
     const int kbegin = zs * g.kchunk;
     const int kend = min(g.K, kbegin + g.kchunk);
     const int ktiles = (kend - kbegin + BK - 1) / BK;
@@ -665,8 +671,17 @@ template <int MODE>
 void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& g, long batch, float* partial)
 {
     dim3 grid((unsigned)(((g.N + 63) / 64) * (long)((g.M + 63) / 64)), (unsigned)p.ksplit, (unsigned)batch);
-    if (p.bk == 32) launch_kinds<32, MODE>(lk, rk, grid, st, g, partial);
-    else launch_kinds<16, MODE>(lk, rk, grid, st, g, partial);
+    // Work-groups go to the eight XCDs in turn, and every XCD has its own L2.  With tiles in launch order the
+    // column tiles of one row tile land on all eight, and each L2 fetches the whole left operand.  For a plain
+    // 2-D product each XCD is given a contiguous range of tiles instead, so it reads only its rows.
+    GemmArgs ga = g;
+    if (p.ksplit == 1 && batch == 1 && grid.x >= 64) {
+        ga.tiles = (int)grid.x;
+        ga.xcd_chunk = (int)((grid.x + 7) / 8);
+        grid.x = (unsigned)(8 * ga.xcd_chunk);
+    }
+    if (p.bk == 32) launch_kinds<32, MODE>(lk, rk, grid, st, ga, partial);
+    else launch_kinds<16, MODE>(lk, rk, grid, st, ga, partial);
 }
 
 int gemm(const char* what, int mode, long batch, long M, long N, long K,
@@ -697,6 +712,7 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     g.bias = bias;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.ksplit = p.ksplit; g.kchunk = p.kchunk;
+    g.xcd_chunk = 0; g.tiles = 0;
     g.off = offset; g.has_off = (mode != MODE_STD && offset != 1.0f) ? 1 : 0;
 
     g.cv = conv ? *conv : ConvGeom{nullptr, nullptr, 0, 0, 0};
