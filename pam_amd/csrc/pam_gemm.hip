@@ -72,7 +72,8 @@ struct GemmArgs {
     const float* bias;           // one value per output column, added once after the sum, or null
     int M, N, K;
     int ksplit, kchunk;          // kchunk is a multiple of 32; ksplit == 1 means no split
-    int xcd_chunk, tiles;        // xcd_chunk > 0: work-group x takes tile (x % 8) * xcd_chunk + x / 8 (see the launch)
+    int tiles, batch;            // output tiles per matrix, matrices
+    long xcd_chunk, units;       // xcd_chunk > 0: a 1-D launch, work-group x takes unit (x % 8) * xcd_chunk + x / 8 (see the launch)
     float off; int has_off;
 };
 
@@ -290,12 +291,14 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 
     const int tid = threadIdx.x, tx = tid % TXN, ty = tid / TXN;
     const int wave = tid / 64, lane = tid % 64;
-    const int zb = blockIdx.z, zs = blockIdx.y;
     const int ntn = (g.N + BN - 1) / BN;                  // consecutive tiles share L rows
-    int tile = blockIdx.x;
-    if (g.xcd_chunk > 0) {                                // one contiguous range of tiles per XCD (its own L2)
-        tile = (int)(blockIdx.x % 8) * g.xcd_chunk + (int)(blockIdx.x / 8);
-        if (tile >= g.tiles) return;                      // the ranges are rounded up: a few work-groups have nothing to do
+    int tile = blockIdx.x, zs = blockIdx.y, zb = blockIdx.z;
+    if (g.xcd_chunk > 0) {                                // units (matrix, k chunk, tile), one contiguous range per XCD
+        const long unit = (long)(blockIdx.x % 8) * g.xcd_chunk + (long)(blockIdx.x / 8);
+        if (unit >= g.units) return;                      // the ranges are rounded up: a few work-groups have nothing to do
+        tile = (int)(unit % g.tiles);
+        const long rest = unit / g.tiles;
+        zs = (int)(rest % g.ksplit); zb = (int)(rest / g.ksplit);
     }
     const int row0 = (tile / ntn) * BM, col0 = (tile % ntn) * BN;
     const int kbegin = zs * g.kchunk;
@@ -511,7 +514,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     // epilogue: to Y, or to this chunk's slab of the split-K scratch ([chunk][batch][M][N])
     float* out; long o_sr, o_sc;
     if (g.ksplit > 1) {
-        out = partial + ((long)zs * gridDim.z + zb) * (long)g.M * g.N; o_sr = g.N; o_sc = 1;
+        out = partial + ((long)zs * g.batch + zb) * (long)g.M * g.N; o_sr = g.N; o_sc = 1;
     } else {
         out = g.Y + (long)zb * g.y_sb; o_sr = g.y_sr; o_sc = g.y_sc;
     }
@@ -672,13 +675,17 @@ void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& 
 {
     dim3 grid((unsigned)(((g.N + 63) / 64) * (long)((g.M + 63) / 64)), (unsigned)p.ksplit, (unsigned)batch);
     // Work-groups go to the eight XCDs in turn, and every XCD has its own L2.  With tiles in launch order the
-    // column tiles of one row tile land on all eight, and each L2 fetches the whole left operand.  For a plain
-    // 2-D product each XCD is given a contiguous range of tiles instead, so it reads only its rows.
+    // column tiles of one row tile land on all eight, and each L2 fetches the whole left operand.  So the launch
+    // is one-dimensional over units (matrix, k chunk, tile) and each XCD is given a contiguous range of them:
+    // it reads only its own rows, chunks and matrices.
     GemmArgs ga = g;
-    if (p.ksplit == 1 && batch == 1 && grid.x >= 64) {
-        ga.tiles = (int)grid.x;
-        ga.xcd_chunk = (int)((grid.x + 7) / 8);
-        grid.x = (unsigned)(8 * ga.xcd_chunk);
+    ga.tiles = (int)grid.x; ga.batch = (int)batch;
+    const long units = (long)grid.x * p.ksplit * batch;
+    // (not for few tiles with many k chunks, the weight-gradient shape: measured 8 % slower that way)
+    if (units >= 64 && units < (1L << 31) - 8 && (p.ksplit == 1 || (long)grid.x >= cu_count())) {
+        ga.units = units;
+        ga.xcd_chunk = (units + 7) / 8;
+        grid = dim3((unsigned)(8 * ga.xcd_chunk), 1, 1);
     }
     if (p.bk == 32) launch_kinds<32, MODE>(lk, rk, grid, st, ga, partial);
     else launch_kinds<16, MODE>(lk, rk, grid, st, ga, partial);
@@ -712,7 +719,7 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     g.bias = bias;
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.ksplit = p.ksplit; g.kchunk = p.kchunk;
-    g.xcd_chunk = 0; g.tiles = 0;
+    g.xcd_chunk = 0; g.units = 0; g.tiles = 0; g.batch = (int)batch;
     g.off = offset; g.has_off = (mode != MODE_STD && offset != 1.0f) ? 1 : 0;
 
     g.cv = conv ? *conv : ConvGeom{nullptr, nullptr, 0, 0, 0};
