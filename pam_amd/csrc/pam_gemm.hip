@@ -7,9 +7,10 @@
 //  * A work-group of four wavefronts owns a 64 x 64 tile of Y.  Each lane owns a 4 x 4
 //    micro-tile in registers, each wavefront 32 x 32 outputs (lanes 8 x 8).  Measured on
 //    MI355X, a SIMD retires a wave64 VALU instruction every two cycles but one wavefront
-//    issues at most one every four, so the design goal is many resident wavefronts (five
-//    per SIMD at under 100 registers) rather than a large micro-tile; thousands of equal
-//    work-groups per product are what balances the 256 compute units.
+//    issues at most one every four, so several wavefronts per SIMD are needed (four are
+//    resident: 104 registers, 35 KB of LDS per work-group with 32-deep k-tiles); larger
+//    micro-tiles and more resident wavefronts were measured and gained nothing.  Thousands
+//    of equal work-groups per product are what balances the 256 compute units.
 //  * L and R tiles are staged through LDS k-major ([k][row], 4-word row pad), so a fragment
 //    for one k is two ds_read_b128, contiguous (R) or broadcast (L) across the wavefront.
 //    Operands whose contiguous dimension is k (row-major L, "column-major" R) are
@@ -28,14 +29,19 @@
 //    in the tile can leave the normal range and the two-instruction loop is exact;
 //    a k-tile that only adds zeros to that in one operand (ReLU activations, padding) keeps two
 //    instructions per product: the zero becomes a stand-in value and the accumulating fma
-//    multiplies the product by 0 or 1; zeros in both operands cost one select per product; anything else (subnormals, inf, NaN, extreme exponents) takes a
-//    guarded loop that evaluates the full definition per product on operands decomposed once
-//    per k-step.  The choice is uniform per work-group and k-tile.
+//    multiplies the product by 0 or 1; zeros in both operands cost one select per product;
+//    anything else (subnormals, inf, NaN, extreme exponents) takes a guarded loop that
+//    evaluates the full definition per product on operands decomposed once per k-step.
+//    The choice is uniform per work-group and k-tile.
 //  * Rows beyond M / N are clamped to the last valid row when loading (their results are
 //    never stored); the k tail runs a shorter loop, padding never enters the arithmetic.
 //  * Shapes with few output tiles and long k (dX: 12608 x 192, k = 768; dW: 192 x 768,
 //    k = 12608) split k across work-groups; the partial tiles go through a scratch buffer
 //    and are added in ascending order by a second kernel.
+//  * The launch is one-dimensional over (matrix, k chunk, tile) units and every XCD (own L2)
+//    takes one contiguous range of them, so each operand is fetched from memory about once.
+//  * The right operand may be the patches of an image read in place (convolutions), and a
+//    bias may be added to the finished sums (linear layers).
 //  * Accumulation order: every output is summed by one lane per k chunk, k ascending, from
 //    +0 -- with one chunk this is the order of the reference kernel
 //    (pam/cuda_kernels.cu:601, 608-627); pam_hip_gemm_plan reports the chunking.
