@@ -127,6 +127,8 @@ def main():
         "frac_of_single_issue_peak": round(2 * macs_each / (head["ms"] * 1e-3) / single_issue_peak, 4),
         "target_in_baseline_plan": ">= 0.60 of the single-issue figure (11.8 T PAM-MAC/s)",
     }
+    # the issue rate of the same instruction mix with register operands only, at 1, 2 and 4 wavefronts per SIMD
+    roofline["register_only_probe_Tlaneop_s"] = {str(w): round(_abi.issue_probe(w), 2) for w in (1, 2, 4)}
     traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
     traffic = json.load(open(traffic_file)) if os.path.exists(traffic_file) else {}
     roofline["traffic"] = traffic.get("gemm_fwd_12608x768x192_bytes")

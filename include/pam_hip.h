@@ -45,6 +45,12 @@ const char *pam_hip_last_error(void);
 /* Compute units and shader clock (kHz) of the current device, for roofline figures. */
 int pam_hip_device_info(int *compute_units, int *clock_khz);
 
+/* Measurement aid, no counterpart in the reference: runs the matrix kernel's instruction mix (one v_add_u32
+ * and one dependent v_add_f32 per product) on register operands only, blocks work-groups of 256 lanes, each lane
+ * iters * 256 VALU lane-operations; timing it gives the vector issue rate the roofline figures are stated against.
+ * seed: 1024 words, out: blocks * 256 floats. */
+int pam_hip_issue_probe(const void *seed, float *out, int blocks, int iters, void *stream);
+
 /* ---- elementwise, n contiguous elements (pam/cuda_kernels.cu:141-328) ------------------ */
 /* C = A (*) B                         replaces pam_fwd  (elementwise_pam_caller,  :155-183) */
 int pam_hip_pam_fwd(const float *a, const float *b, float *c, size_t n, float offset, void *stream);

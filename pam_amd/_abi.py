@@ -33,6 +33,7 @@ _SIGNATURES = {
     "pam_hip_pad_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
     "pam_hip_pa_exp_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_exp_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
+    "pam_hip_issue_probe": ([_p, _p, _i, _i, _p], _i),
     "pam_hip_pam_bwd_pair": ([_p, _p, _p, _p, _p, _z, _f, _i, _i, _p], _i),
     "pam_hip_pad_bwd_pair": ([_p, _p, _p, _p, _p, _z, _f, _i, _i, _p], _i),
     "pam_hip_pow_fwd": ([_p, _p, _z, _f, _f, _p], _i),
@@ -422,6 +423,22 @@ class HipRowKernels:
                 _call("pam_hip_layer_norm_fwd", X.data_ptr(), None if weight is None else weight.data_ptr(),
                       None if bias is None else bias.data_ptr(), Y.data_ptr(), rows, n, float(eps), float(offset), _stream())
         return Y
+
+
+def issue_probe(work_groups_per_cu, iters=400):
+    """T lane-operations per second of register-only product-accumulate pairs with that many 256-lane
+    work-groups per compute unit (= wavefronts per SIMD)."""
+    cus, _ = device_info()
+    blocks = cus * work_groups_per_cu
+    seed = torch.full((1024,), 2.0 ** -20, dtype=torch.float32, device="cuda")
+    out = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    _call("pam_hip_issue_probe", seed.data_ptr(), out.data_ptr(), blocks, 5, _stream())
+    torch.cuda.synchronize()
+    start.record()
+    _call("pam_hip_issue_probe", seed.data_ptr(), out.data_ptr(), blocks, iters, _stream())
+    stop.record(); stop.synchronize()
+    return blocks * 256.0 * iters * 256 / (start.elapsed_time(stop) * 1e-3) / 1e12
 
 
 def pow_fwd(X, exponent, offset):

@@ -353,9 +353,53 @@ __global__ __launch_bounds__(kThreads) void adam_scalar_kernel(float* __restrict
     }
 }
 
+// Measures what the vector ALUs issue on the matrix kernel's instruction mix with nothing else in the way:
+// per lane 4 x 8 accumulators, and per product one v_add_u32 and one v_add_f32 that depends on it, operands in
+// registers, no memory traffic.  The empty asm statements keep the compiler from hoisting the integer adds.
+__global__ __launch_bounds__(kThreads) void issue_probe_kernel(const uint32_t* __restrict__ seed, float* __restrict__ out, int iters)
+{
+    const int lane = threadIdx.x;
+    float acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = 0.0f;
+    uint32_t a[4], b[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] = seed[(lane + i) & 1023];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) b[j] = seed[(lane * 3 + j) & 1023];
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(a[i]));
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[i][j] += u2f(a[i] + b[j]);
+        }
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) total += acc[i][j];
+    out[(size_t)blockIdx.x * kThreads + lane] = total;
+}
+
 }  // namespace
 
 extern "C" {
+
+// seed: 1024 words (any bit patterns of normal numbers), out: blocks * 256 floats; each lane executes
+// iters * 4 * 32 product-accumulate pairs = iters * 256 VALU lane-operations
+int pam_hip_issue_probe(const void* seed, float* out, int blocks, int iters, void* stream)
+{
+    if (!seed || !out || blocks <= 0 || iters < 0) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "issue_probe: bad argument");
+    hipLaunchKernelGGL(issue_probe_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint32_t*)seed, out, iters);
+    return pamhost::check_launch("issue_probe");
+}
 
 int pam_hip_abi_version(void) { return PAM_HIP_ABI_VERSION; }
 const char* pam_hip_last_error(void) { return pamhost::error_buffer(); }
