@@ -128,7 +128,9 @@ def main():
         "target_in_baseline_plan": ">= 0.60 of the single-issue figure (11.8 T PAM-MAC/s)",
     }
     # the issue rate of the same instruction mix with register operands only, at 1, 2 and 4 wavefronts per SIMD
-    roofline["register_only_probe_Tlaneop_s"] = {str(w): round(_abi.issue_probe(w), 2) for w in (1, 2, 4)}
+    roofline["register_only_probe_Tlaneop_s"] = {str(w): round(_abi.issue_probe(w), 2) for w in (1, 2, 4, 8)}
+    # and with every step's operands read from LDS the way the kernel's inner loop reads them (4 x 4 per lane)
+    roofline["lds_fed_4x4_probe_Tlaneop_s"] = {str(w): round(_abi.issue_probe(w, lds_tile=(4, 4)), 2) for w in (1, 2, 4, 8)}
     traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
     traffic = json.load(open(traffic_file)) if os.path.exists(traffic_file) else {}
     roofline["traffic"] = traffic.get("gemm_fwd_12608x768x192_bytes")

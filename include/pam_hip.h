@@ -50,6 +50,9 @@ int pam_hip_device_info(int *compute_units, int *clock_khz);
  * iters * 256 VALU lane-operations; timing it gives the vector issue rate the roofline figures are stated against.
  * seed: 1024 words, out: blocks * 256 floats. */
 int pam_hip_issue_probe(const void *seed, float *out, int blocks, int iters, void *stream);
+/* The same with every step's operands read from LDS as the matrix kernel's inner loop reads them, for a
+ * tm x tn micro-tile (4x4, 8x4, 8x8); each lane iters * 32 * tm * tn pairs. */
+int pam_hip_issue_probe_lds(const void *seed, float *out, int blocks, int iters, int tm, int tn, void *stream);
 
 /* ---- elementwise, n contiguous elements (pam/cuda_kernels.cu:141-328) ------------------ */
 /* C = A (*) B                         replaces pam_fwd  (elementwise_pam_caller,  :155-183) */

@@ -34,6 +34,7 @@ _SIGNATURES = {
     "pam_hip_pa_exp_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_exp_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
     "pam_hip_issue_probe": ([_p, _p, _i, _i, _p], _i),
+    "pam_hip_issue_probe_lds": ([_p, _p, _i, _i, _i, _i, _p], _i),
     "pam_hip_pam_bwd_pair": ([_p, _p, _p, _p, _p, _z, _f, _i, _i, _p], _i),
     "pam_hip_pad_bwd_pair": ([_p, _p, _p, _p, _p, _z, _f, _i, _i, _p], _i),
     "pam_hip_pow_fwd": ([_p, _p, _z, _f, _f, _p], _i),
@@ -425,20 +426,31 @@ class HipRowKernels:
         return Y
 
 
-def issue_probe(work_groups_per_cu, iters=400):
-    """T lane-operations per second of register-only product-accumulate pairs with that many 256-lane
-    work-groups per compute unit (= wavefronts per SIMD)."""
+def issue_probe(work_groups_per_cu, iters=400, lds_tile=None):
+    """T lane-operations per second of product-accumulate pairs (v_add_u32 + dependent v_add_f32) with that many
+    256-lane work-groups per compute unit (= wavefronts per SIMD): operands in registers, or, with
+    lds_tile=(tm, tn), read from LDS per step as the matrix kernel's inner loop reads them."""
     cus, _ = device_info()
     blocks = cus * work_groups_per_cu
     seed = torch.full((1024,), 2.0 ** -20, dtype=torch.float32, device="cuda")
     out = torch.empty(blocks * 256, dtype=torch.float32, device="cuda")
+
+    def launch(n):
+        if lds_tile is None:
+            _call("pam_hip_issue_probe", seed.data_ptr(), out.data_ptr(), blocks, n, _stream())
+        else:
+            _call("pam_hip_issue_probe_lds", seed.data_ptr(), out.data_ptr(), blocks, n, lds_tile[0], lds_tile[1], _stream())
+
+    pairs = 128 if lds_tile is None else 32 * lds_tile[0] * lds_tile[1]
+    if lds_tile is not None:
+        iters = max(1, iters * 128 // pairs)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    _call("pam_hip_issue_probe", seed.data_ptr(), out.data_ptr(), blocks, 5, _stream())
+    launch(2)
     torch.cuda.synchronize()
     start.record()
-    _call("pam_hip_issue_probe", seed.data_ptr(), out.data_ptr(), blocks, iters, _stream())
+    launch(iters)
     stop.record(); stop.synchronize()
-    return blocks * 256.0 * iters * 256 / (start.elapsed_time(stop) * 1e-3) / 1e12
+    return blocks * 256.0 * iters * pairs * 2 / (start.elapsed_time(stop) * 1e-3) / 1e12
 
 
 def pow_fwd(X, exponent, offset):
