@@ -574,3 +574,27 @@ def test_degenerate_shapes(K, oracle):
         pam_amd.softmax(z(4, 0), dim=-1)
     assert _abi.conv2d_fwd(z(0, 3, 8, 8), z(4, 3, 3, 3), (1, 1), (1, 1), 1.0).shape == (0, 4, 8, 8)
     assert K.pam_fwd(z(0), z(0), 1.0).shape == (0,)
+
+
+def test_more_than_two_to_the_31_elements(K, oracle):
+    """64-bit indexing: an elementwise product over 2^31 + 5 elements, a row kernel over 2^31 elements and a product
+    with more than 2^31 output elements, checked on slices from both ends."""
+    from pam_amd import _abi
+    n = (1 << 31) + 5
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.randn(n, device="cuda", generator=gen); b = torch.randn(n, device="cuda", generator=gen)
+    c = K.pam_fwd(a, b, 1.0)
+    for lo, hi in ((0, 4096), (n - 4101, n)):
+        assert_same_bits(host(c[lo:hi]), oracle.pam(host(a[lo:hi]), host(b[lo:hi])), f"elementwise [{lo}:{hi}]")
+    del c, b
+    rows = a[:1 << 31].view(1 << 21, 1024)
+    R = _abi.HipRowKernels()
+    y = R.layer_norm_fwd(rows, None, None, 1e-5, 1.0)
+    for lo, hi in ((0, 3), ((1 << 21) - 3, 1 << 21)):
+        assert_same_bits(host(y[lo:hi]), oracle.layer_norm_fwd(host(rows[lo:hi]), None, None, 1e-5, None), f"layer_norm rows [{lo}:{hi}]")
+    del y
+    m = (1 << 25) + 64                                  # m x 64 outputs > 2^31
+    L = a[:m * 16].view(m, 16); Rm = torch.randn(16, 64, device="cuda", generator=gen)
+    Y = K.pam_matmul_fwd(L, Rm, True, True, 1.0)
+    for lo, hi in ((0, 70), (m - 70, m)):
+        assert_same_bits(host(Y[lo:hi]), ogemm(oracle, host(L[lo:hi]), host(Rm), plan_shape=(1, m, 64, 16)), f"product rows [{lo}:{hi}]")
