@@ -46,6 +46,7 @@
 //    +0 -- with one chunk this is the order of the reference kernel
 //    (pam/cuda_kernels.cu:601, 608-627); pam_hip_gemm_plan reports the chunking.
 #include <cmath>
+#include <cstring>
 
 #include "pam_common.h"
 #include "pam_device.h"
@@ -80,7 +81,8 @@ struct GemmArgs {
     int ksplit, kchunk;          // kchunk is a multiple of 32; ksplit == 1 means no split
     int tiles, batch;            // output tiles per matrix, matrices
     long xcd_chunk, units;       // xcd_chunk > 0: a 1-D launch, work-group x takes unit (x % 8) * xcd_chunk + x / 8 (see the launch)
-    float off; int has_off;
+    float off; int has_off;      // has_off: 0 none, 1 a normal number (off_add = its bit-pattern increment), 2 any other value
+    uint32_t off_add;
 };
 
 // Classifies and transforms one staged value.  MODE_PAM: R carries the bias subtraction, and
@@ -122,6 +124,20 @@ struct Stager {
     // some staged value lies outside [2^-63, 2^64) or is not a normal number or zero
     __device__ __forceinline__ bool out_of_range() const { return bad || emin < 64u || emax > 190u; }
 };
+
+// Staging when the quick test below has passed: every value of the k-tile is a normal number in
+// [2^-63, 2^64), so the transformed value is an integer add (the bias subtraction and a normal offset).
+template <bool ADDS>
+struct PlainStager {
+    uint32_t add;
+    __device__ __forceinline__ uint32_t one(float v) const { return ADDS ? f2u(v) + add : f2u(v); }
+};
+
+// Quick test of a staged value: (bits << 1) - (64 << 24) is below 127 << 24 exactly for the normal numbers
+// with biased exponent 64 ... 190, whatever the sign.  One shift-add per value, the results folded by max.
+constexpr uint32_t kWindowBase = 0u - (64u << 24), kWindowSpan = 127u << 24;
+__device__ __forceinline__ uint32_t window(uint32_t u) { return (u << 1) + kWindowBase; }
+__device__ __forceinline__ uint32_t max3u(uint32_t a, uint32_t b, uint32_t c) { return max(max(a, b), c); }
 
 // Verdict of a k-tile: bit 0 / bit 1 = the left / right operand holds zeros (all else in range),
 // kGuarded = some value needs the full definition.  Verdicts of wavefronts combine by OR.
@@ -197,6 +213,24 @@ struct TileLoader {
                 s[i] = base[(long)row * op.sr + (long)kk * op.sk];
             }
         }
+    }
+
+    // max over the tile's values of window(bits), and of window(bits + add) too when `shifted`
+    // (an operand that takes a normal offset must be in range before and after it)
+    __device__ __forceinline__ uint32_t window_max(bool shifted, uint32_t add) const
+    {
+        constexpr int n = (KIND == LOAD_KVEC || KIND == LOAD_RVEC) ? 4 * kVecs : kElems;
+        const float* s = reinterpret_cast<const float*>(v);
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i + 1 < n; i += 2) m = max3u(m, window(f2u(s[i])), window(f2u(s[i + 1])));
+        if (n % 2) m = max(m, window(f2u(s[n - 1])));
+        if (shifted) {
+#pragma unroll
+            for (int i = 0; i + 1 < n; i += 2) m = max3u(m, window(f2u(s[i]) + add), window(f2u(s[i + 1]) + add));
+            if (n % 2) m = max(m, window(f2u(s[n - 1]) + add));
+        }
+        return m;
     }
 
     // R' = R (*) offset, once per element (uniform branch around the whole tile)
@@ -277,6 +311,35 @@ __device__ __forceinline__ uint32_t normalised_fraction(float d)
     return m;
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef const __attribute__((address_space(3))) u32x4* LdsVec;
+
+// 16 PAM products of a 4 x 4 micro-tile added to their accumulators: v_add_u32 + v_add_f32 each, the integer add
+// of the next product issued ahead of the float add of the current one.  Written out because the compiler, given
+// the unrolled k-tile as one block, moves all of its LDS reads to the top and spills; the LDS addresses pass
+// through (unchanged) so that the reads of the step after next cannot be issued before this block.
+__device__ __forceinline__ void pam_mac_4x4(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
+{
+    uint32_t t0, t1;
+#define PAM_MAC_ROW(I)                                              \
+    "v_add_u32 %[t1], %[a" #I "], %[b1]\n v_add_f32 %[c" #I "0], %[c" #I "0], %[t0]\n" \
+    "v_add_u32 %[t0], %[a" #I "], %[b2]\n v_add_f32 %[c" #I "1], %[c" #I "1], %[t1]\n" \
+    "v_add_u32 %[t1], %[a" #I "], %[b3]\n v_add_f32 %[c" #I "2], %[c" #I "2], %[t0]\n"
+    asm volatile(
+        "v_add_u32 %[t0], %[a0], %[b0]\n"
+        PAM_MAC_ROW(0) "v_add_u32 %[t0], %[a1], %[b0]\n v_add_f32 %[c03], %[c03], %[t1]\n"
+        PAM_MAC_ROW(1) "v_add_u32 %[t0], %[a2], %[b0]\n v_add_f32 %[c13], %[c13], %[t1]\n"
+        PAM_MAC_ROW(2) "v_add_u32 %[t0], %[a3], %[b0]\n v_add_f32 %[c23], %[c23], %[t1]\n"
+        PAM_MAC_ROW(3) "v_add_f32 %[c33], %[c33], %[t1]\n"
+        : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),
+          [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
+          [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),
+          [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
+          [t0] "=&v"(t0), [t1] "=&v"(t1), [pl] "+v"(pl), [pr] "+v"(pr)
+        : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+#undef PAM_MAC_ROW
+}
+
 #ifdef PAM_GEMM_WAVES
 #define PAM_GEMM_OCCUPANCY __attribute__((amdgpu_waves_per_eu(PAM_GEMM_WAVES)))
 #else
@@ -339,6 +402,24 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     TileLoader<BN, NT, RKIND, BK> rl;
 
     auto stage = [&](int buf) {
+        PlainStager<false> same{0u};
+        if (MODE == MODE_STD) {
+            ll.store(lds_l[buf], tid, same);
+            rl.store(lds_r[buf], tid, same);
+            return;
+        }
+        // Quick test first: nearly every k-tile holds only normal numbers of moderate size, and then staging is
+        // the shift-add and max per value below plus an integer add for the operand that carries the bias.
+        constexpr bool kOffL = Stager<MODE, false>::kTakesOffset, kOffR = Stager<MODE, true>::kTakesOffset;
+        const bool shifted = g.has_off == 1;
+        const uint32_t worst = max(ll.window_max(kOffL && shifted, g.off_add), rl.window_max(kOffR && shifted, g.off_add));
+        if (__builtin_expect(__ballot(worst >= kWindowSpan) == 0ull && g.has_off != 2, 1)) {
+            PlainStager<true> plus{(MODE == MODE_PAM ? 0u - kBias : 0u) + (shifted ? g.off_add : 0u)};
+            if (kOffL && (MODE == MODE_PAM || shifted)) ll.store(lds_l[buf], tid, plus); else ll.store(lds_l[buf], tid, same);
+            if (kOffR && (MODE == MODE_PAM || shifted)) rl.store(lds_r[buf], tid, plus); else rl.store(lds_r[buf], tid, same);
+            if (lane == 0) lds_flag[buf][wave] = 0u;
+            return;
+        }
         Stager<MODE, false> sl; Stager<MODE, true> sr;
         if (has_off) {
             if (Stager<MODE, false>::kTakesOffset) ll.apply_offset(g.off);
@@ -346,11 +427,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         }
         ll.store(lds_l[buf], tid, sl);
         rl.store(lds_r[buf], tid, sr);
-        if (MODE != MODE_STD) {
-            const uint32_t found = (__ballot(sl.out_of_range() || sr.out_of_range()) != 0ull ? kGuarded : 0u)
-                                 | (__ballot(sl.zero) != 0ull ? kZerosL : 0u) | (__ballot(sr.zero) != 0ull ? kZerosR : 0u);
-            if (lane == 0) lds_flag[buf][wave] = found;
-        }
+        const uint32_t found = (__ballot(sl.out_of_range() || sr.out_of_range()) != 0ull ? kGuarded : 0u)
+                             | (__ballot(sl.zero) != 0ull ? kZerosL : 0u) | (__ballot(sr.zero) != 0ull ? kZerosR : 0u);
+        if (lane == 0) lds_flag[buf][wave] = found;
     };
 
     if (ktiles > 0) {
@@ -360,7 +439,11 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     }
     __syncthreads();
 
-    for (int t = 0; t < ktiles; ++t) {
+    // per k-tile: where its fragments are in LDS, how many k it holds, and what the staging found in it
+    const uint32_t* sl = nullptr; const uint32_t* sr = nullptr;
+    int kcount = 0;
+    uint32_t verdict = 0;                         // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
+    auto begin_tile = [&](int t) {
         const int cur = t & 1;
         const int k0 = kbegin + t * BK;
         // The next tile is fetched unconditionally: past the end the clamped addresses re-read the last
@@ -368,137 +451,168 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         // contents and make the compiler wait for the data right here.
         ll.load(g.L, lbase, row0, g.M, k0 + BK, kend, tid, g.cv);
         rl.load(g.R, rbase, col0, g.N, k0 + BK, kend, tid, g.cv);
-        const int kcount = min(BK, kend - k0);
-        uint32_t verdict = 0;                     // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
+        kcount = min(BK, kend - k0);
         if (MODE != MODE_STD) {
             uint32_t f = 0;
 #pragma unroll
             for (int w = 0; w < NW; ++w) f |= lds_flag[cur][w];
             verdict = __builtin_amdgcn_readfirstlane(f);
         }
-        const uint32_t* sl = lds_l[cur] + ty * 4;
-        const uint32_t* sr = lds_r[cur] + tx * 4;
+        sl = lds_l[cur] + ty * 4;
+        sr = lds_r[cur] + tx * 4;
+    };
+    auto end_tile = [&](int t) {
+        if (t + 1 < ktiles) stage((t & 1) ^ 1);
+        __syncthreads();
+    };
 
-        auto fragment = [&](int kk, uint32_t (&a)[TM], uint32_t (&b)[TN]) {
+    auto fragment = [&](int kk, uint32_t (&a)[TM], uint32_t (&b)[TN]) {
 #pragma unroll
-            for (int gi = 0; gi < GM; ++gi) {
-                uint4 q = *reinterpret_cast<const uint4*>(sl + kk * LDL + gi * (BM / GM));
-                a[gi * 4 + 0] = q.x; a[gi * 4 + 1] = q.y; a[gi * 4 + 2] = q.z; a[gi * 4 + 3] = q.w;
-            }
+        for (int gi = 0; gi < GM; ++gi) {
+            uint4 q = *reinterpret_cast<const uint4*>(sl + kk * LDL + gi * (BM / GM));
+            a[gi * 4 + 0] = q.x; a[gi * 4 + 1] = q.y; a[gi * 4 + 2] = q.z; a[gi * 4 + 3] = q.w;
+        }
 #pragma unroll
-            for (int gj = 0; gj < GN; ++gj) {
-                uint4 q = *reinterpret_cast<const uint4*>(sr + kk * LDR + gj * (BN / GN));
-                b[gj * 4 + 0] = q.x; b[gj * 4 + 1] = q.y; b[gj * 4 + 2] = q.z; b[gj * 4 + 3] = q.w;
-            }
-        };
-        auto fast_step = [&](int kk) {
-            uint32_t a[TM], b[TN];
-            fragment(kk, a, b);
+        for (int gj = 0; gj < GN; ++gj) {
+            uint4 q = *reinterpret_cast<const uint4*>(sr + kk * LDR + gj * (BN / GN));
+            b[gj * 4 + 0] = q.x; b[gj * 4 + 1] = q.y; b[gj * 4 + 2] = q.z; b[gj * 4 + 3] = q.w;
+        }
+    };
+    auto fast_step = [&](int kk) {
+        uint32_t a[TM], b[TN];
+        fragment(kk, a, b);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    if (MODE == MODE_PAM) acc[i][j] += u2f(a[i] + b[j]);
-                    else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(a[i]), u2f(b[j]), acc[i][j]);
-                    else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(a[i]), u2f((b[j] + dfrac[i][j]) & ~kMant), acc[i][j]);
-                    else acc[i][j] = fmaf(u2f(b[j]), u2f((a[i] + dfrac[i][j]) & ~kMant), acc[i][j]);
-                }
-        };
-        // k-tile with zeros but otherwise in range: the integer add of a zero is garbage, so those
-        // products are replaced by +0 (one v_cndmask per product, masks combined on the scalar unit)
-        auto zeros_step = [&](int kk) {
-            uint32_t a[TM], b[TN];
-            fragment(kk, a, b);
-            bool za[TM], zb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) za[i] = a[i] == kZeroL;
-#pragma unroll
-            for (int j = 0; j < TN; ++j) zb[j] = b[j] == kZeroR;
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] += u2f((za[i] | zb[j]) ? 0u : a[i] + b[j]);
-        };
-        // zeros in one operand only: its zeros become a stand-in that keeps the integer sum finite, and
-        // the product is multiplied by 0 or 1 in the accumulating fma (x * 1 + acc rounds like acc + x;
-        // x * 0 + acc leaves acc, which is never -0) -- two instructions per product like the plain loop,
-        // plus three per value of the operand with zeros
-        auto zeros_left_step = [&](int kk) {
-            uint32_t a[TM], b[TN];
-            fragment(kk, a, b);
-            float keep[TM];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const uint64_t nonzero = __ballot(a[i] != kZeroL);
-                keep[i] = u2f(pick(nonzero, 0u, 0x3f800000u));
-                a[i] = max(a[i], kStandInL);          // every other value is larger, as an unsigned number
-            }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[i], acc[i][j]);
-        };
-        auto zeros_right_step = [&](int kk) {
-            uint32_t a[TM], b[TN];
-            fragment(kk, a, b);
-            float keep[TN];
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const uint64_t nonzero = __ballot(b[j] != kZeroR);
-                keep[j] = u2f(pick(nonzero, 0u, 0x3f800000u));
-                b[j] = pick(nonzero, kStandInR, b[j]);
+                if (MODE == MODE_PAM) acc[i][j] += u2f(a[i] + b[j]);
+                else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(a[i]), u2f(b[j]), acc[i][j]);
+                else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(a[i]), u2f((b[j] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                else acc[i][j] = fmaf(u2f(b[j]), u2f((a[i] + dfrac[i][j]) & ~kMant), acc[i][j]);
             }
+    };
+    // k-tile with zeros but otherwise in range: the integer add of a zero is garbage, so those
+    // products are replaced by +0 (one v_cndmask per product, masks combined on the scalar unit)
+    auto zeros_step = [&](int kk) {
+        uint32_t a[TM], b[TN];
+        fragment(kk, a, b);
+        bool za[TM], zb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) za[i] = a[i] == kZeroL;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) zb[j] = b[j] == kZeroR;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] += u2f((za[i] | zb[j]) ? 0u : a[i] + b[j]);
+    };
+    // zeros in one operand only: its zeros become a stand-in that keeps the integer sum finite, and
+    // the product is multiplied by 0 or 1 in the accumulating fma (x * 1 + acc rounds like acc + x;
+    // x * 0 + acc leaves acc, which is never -0) -- two instructions per product like the plain loop,
+    // plus three per value of the operand with zeros
+    auto zeros_left_step = [&](int kk) {
+        uint32_t a[TM], b[TN];
+        fragment(kk, a, b);
+        float keep[TM];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const uint64_t nonzero = __ballot(a[i] != kZeroL);
+            keep[i] = u2f(pick(nonzero, 0u, 0x3f800000u));
+            a[i] = max(a[i], kStandInL);          // every other value is larger, as an unsigned number
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[i], acc[i][j]);
+    };
+    auto zeros_right_step = [&](int kk) {
+        uint32_t a[TM], b[TN];
+        fragment(kk, a, b);
+        float keep[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const uint64_t nonzero = __ballot(b[j] != kZeroR);
+            keep[j] = u2f(pick(nonzero, 0u, 0x3f800000u));
+            b[j] = pick(nonzero, kStandInR, b[j]);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[j], acc[i][j]);
+    };
+    auto guarded_step = [&](int kk) {
+        uint32_t a[TM], b[TN];
+        fragment(kk, a, b);
+        if (MODE == MODE_PAM) {
+            Split sa[TM], sb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) sa[i] = split_operand(a[i], 127);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) sb[j] = split_operand(b[j] + kBias, 0);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[j], acc[i][j]);
-        };
-        auto guarded_step = [&](int kk) {
-            uint32_t a[TM], b[TN];
-            fragment(kk, a, b);
-            if (MODE == MODE_PAM) {
-                Split sa[TM], sb[TN];
+                for (int j = 0; j < TN; ++j) acc[i][j] += pam_from_split(sa[i], sb[j]);
+            return;
+        }
 #pragma unroll
-                for (int i = 0; i < TM; ++i) sa[i] = split_operand(a[i], 127);
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) sb[j] = split_operand(b[j] + kBias, 0);
+            for (int j = 0; j < TN; ++j) {
+                if (MODE == MODE_BWD_DL) acc[i][j] += bwd_product_general(dfrac[i][j], b[j], u2f(a[i]));
+                else if (MODE == MODE_BWD_DR) acc[i][j] += bwd_product_general(dfrac[i][j], a[i], u2f(b[j]));
+            }
+    };
+
+    // a full k-tile of in-range values: fragments for step kk+1 are read from LDS while step kk is computed
+    auto plain_tile = [&]() {
+        if constexpr (MODE == MODE_PAM && TM == 4 && TN == 4) {
+            typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
+            uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            u32x4 fa[2], fb[2];
+            fa[0] = *reinterpret_cast<LdsVec>(pl); fb[0] = *reinterpret_cast<LdsVec>(pr);
+#pragma unroll
+            for (int kk = 0; kk < BK; ++kk) {
+                if (kk + 1 < BK) {
+                    fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
+                    fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
+                }
+                pam_mac_4x4(acc, fa[kk & 1], fb[kk & 1], pl, pr);
+            }
+        } else {
+            uint32_t fa[2][TM], fb[2][TN];
+            fragment(0, fa[0], fb[0]);
+#pragma unroll
+            for (int kk = 0; kk < BK; ++kk) {
+                if (kk + 1 < BK) fragment(kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] += pam_from_split(sa[i], sb[j]);
-                return;
+                    for (int j = 0; j < TN; ++j) {
+                        if (MODE == MODE_PAM) acc[i][j] += u2f(fa[kk & 1][i] + fb[kk & 1][j]);
+                        else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f(fb[kk & 1][j]), acc[i][j]);
+                        else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f((fb[kk & 1][j] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                        else acc[i][j] = fmaf(u2f(fb[kk & 1][j]), u2f((fa[kk & 1][i] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                    }
             }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    if (MODE == MODE_BWD_DL) acc[i][j] += bwd_product_general(dfrac[i][j], b[j], u2f(a[i]));
-                    else if (MODE == MODE_BWD_DR) acc[i][j] += bwd_product_general(dfrac[i][j], a[i], u2f(b[j]));
-                }
-        };
+        }
+    };
 
-        if (__builtin_expect(verdict == 0, 1)) {
-            if (kcount == BK) {
-                // fragments for step kk+1 are read from LDS while step kk is computed
-                uint32_t fa[2][TM], fb[2][TN];
-                fragment(0, fa[0], fb[0]);
-#pragma unroll
-                for (int kk = 0; kk < BK; ++kk) {
-                    if (kk + 1 < BK) fragment(kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-#pragma unroll
-                    for (int i = 0; i < TM; ++i)
-#pragma unroll
-                        for (int j = 0; j < TN; ++j) {
-                            if (MODE == MODE_PAM) acc[i][j] += u2f(fa[kk & 1][i] + fb[kk & 1][j]);
-                            else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f(fb[kk & 1][j]), acc[i][j]);
-                            else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f((fb[kk & 1][j] + dfrac[i][j]) & ~kMant), acc[i][j]);
-                            else acc[i][j] = fmaf(u2f(fb[kk & 1][j]), u2f((fa[kk & 1][i] + dfrac[i][j]) & ~kMant), acc[i][j]);
-                        }
-                }
-            } else {
+    int t = 0;
+    while (t < ktiles) {
+        begin_tile(t);
+        // Runs of full plain k-tiles -- nearly all of them -- are a loop of their own: the accumulators then stay
+        // in the same registers from one k-tile to the next instead of being moved to where the other loops want them.
+        while (verdict == 0 && kcount == BK) {
+            plain_tile();
+            end_tile(t);
+            if (++t == ktiles) break;
+            begin_tile(t);
+        }
+        if (t == ktiles) break;
+        if (verdict == 0) {
 #pragma unroll 1
-                for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
-            }
+            for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
         } else if (verdict == kZerosL && MODE == MODE_PAM) {
 #pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) zeros_left_step(kk);
@@ -512,9 +626,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 #pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) guarded_step(kk);
         }
-
-        if (t + 1 < ktiles) stage(cur ^ 1);
-        __syncthreads();
+        end_tile(t);
+        ++t;
     }
 
     // epilogue: to Y, or to this chunk's slab of the split-K scratch ([chunk][batch][M][N])
@@ -667,8 +780,12 @@ void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, 
 {
 #define PAM_GEMM_CASE(LK, RK) \
     if (lk == LK && rk == RK) { hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 4, BK, MODE, LK, RK>), grid, dim3(256), 0, st, g, partial); return; }
-    PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
-    PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
+    PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC)
+#ifdef PAM_GEMM_FEW
+    return;
+#endif
+    PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
+    PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
     if constexpr (MODE != MODE_STD) {                                  // image patches as the right operand
         PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_RVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_ANY, LOAD_CONV)
@@ -726,7 +843,12 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     g.M = (int)M; g.N = (int)N; g.K = (int)K;
     g.ksplit = p.ksplit; g.kchunk = p.kchunk;
     g.xcd_chunk = 0; g.units = 0; g.tiles = 0; g.batch = (int)batch;
-    g.off = offset; g.has_off = (mode != MODE_STD && offset != 1.0f) ? 1 : 0;
+    g.off = offset; g.off_add = 0; g.has_off = 0;
+    if (mode != MODE_STD && offset != 1.0f) {
+        uint32_t bits; memcpy(&bits, &offset, sizeof bits);
+        g.has_off = std::isnormal(offset) ? 1 : 2;
+        g.off_add = bits - kBias;
+    }
 
     g.cv = conv ? *conv : ConvGeom{nullptr, nullptr, 0, 0, 0};
 
@@ -735,9 +857,13 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     float* partial = (float*)workspace;
     switch (mode) {
     case MODE_PAM: launch_mode<MODE_PAM>(p, lk, rk, st, g, batch, partial); break;
+#ifndef PAM_GEMM_FEW
     case MODE_STD: launch_mode<MODE_STD>(p, lk, rk, st, g, batch, partial); break;
     case MODE_BWD_DL: launch_mode<MODE_BWD_DL>(p, lk, rk, st, g, batch, partial); break;
     default: launch_mode<MODE_BWD_DR>(p, lk, rk, st, g, batch, partial); break;
+#else
+    default: return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: experimental build without this mode", what);
+#endif
     }
     if (p.ksplit > 1) {
         long slab = batch * M * N;
