@@ -118,6 +118,16 @@ int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_chunk, int *k_g
 int pam_hip_pam_matmul_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
                            float *y, long y_sr, long y_sc, long m, long n, long k, float offset,
                            void *workspace, size_t workspace_bytes, void *stream);
+/* The same product for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The split-k partial tiles go to an
+ * array of PAM_HIP_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, for the life of
+ * the process; the call allocates and frees nothing.  Results are bit-identical to pam_hip_pam_matmul_fwd with
+ * a workspace of pam_hip_gemm_workspace_bytes(1, m, n, k).  A shape that needs more scratch than the array is
+ * refused with PAM_HIP_ERR_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on the
+ * same GPU (different streams or threads) race, so serialise them. */
+#define PAM_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+int pam_hip_pam_matmul_fwd_noalloc(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
+                                   float *y, long y_sr, long y_sc, long m, long n, long k, float offset, void *stream);
 /* Y = A (x) B + bias[column]: the product followed by the bias add of pam.linear
  * (pam/pam_ops.py:107-115) in one pass; the bias is added once to the finished sum (after the chunk
  * sums when k is split), which is what the separate add computes.  bias NULL = no bias. */

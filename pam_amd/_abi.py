@@ -44,6 +44,7 @@ _SIGNATURES = {
     "pam_hip_gemm_workspace_bytes": ([_l, _l, _l, _l], _z),
     "pam_hip_gemm_plan": ([_l, _l, _l, _l, ctypes.POINTER(_i), ctypes.POINTER(_i)], _i),
     "pam_hip_pam_matmul_fwd": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),
+    "pam_hip_pam_matmul_fwd_noalloc": (_MAT2 * 3 + [_l, _l, _l, _f, _p], _i),
     "pam_hip_pam_linear_fwd": (_MAT2 * 2 + [_p] + _MAT2 + [_l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_bmm_fwd": (_MAT * 3 + [_l, _l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_standard_matmul": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),

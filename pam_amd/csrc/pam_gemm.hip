@@ -47,6 +47,7 @@
 //    (pam/cuda_kernels.cu:601, 608-627); pam_hip_gemm_plan reports the chunking.
 #include <cmath>
 #include <cstring>
+#include <mutex>
 
 #include "pam_common.h"
 #include "pam_device.h"
@@ -988,6 +989,36 @@ ConvSpace input_gradient_space(const ConvShape& t)
     return w;
 }
 
+// ---------------------------------------------------------------- scratch that the library owns
+// For callers that cannot allocate (code under graph capture, serving loops, harnesses that forbid hipMalloc):
+// the split-k partial tiles of pam_hip_pam_matmul_fwd_noalloc go to this array instead of a workspace argument.
+// Every GPU the library runs on holds its own copy, at its own address, until the process ends.
+constexpr size_t kScratchBytes = (size_t)PAM_HIP_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// The array's address on the current device.  In host code `scratch` is only a stand-in for the symbol, never an
+// address to hand to a kernel; the address is looked up once per device, with that device current.
+int scratch_address(const char* what, void** ptr)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return pamhost::fail(PAM_HIP_ERR_LAUNCH, "%s: hipGetDevice: %s", what, hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: device %d beyond the %d this entry point keeps scratch for", what, dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return pamhost::fail(PAM_HIP_ERR_LAUNCH, "%s: hipGetSymbolAddress: %s", what, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return PAM_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1016,6 +1047,22 @@ int pam_hip_pam_matmul_fwd(const float* a, long a_sr, long a_sc, const float* b,
 {
     return gemm("pam_matmul_fwd", MODE_PAM, 1, m, n, k, a, 0, a_sr, a_sc, b, 0, b_sr, b_sc, nullptr, 0, 0, 0,
                 y, 0, y_sr, y_sc, offset, workspace, workspace_bytes, stream);
+}
+
+int pam_hip_pam_matmul_fwd_noalloc(const float* a, long a_sr, long a_sc, const float* b, long b_sr, long b_sc,
+                                   float* y, long y_sr, long y_sc, long m, long n, long k, float offset, void* stream)
+{
+    const size_t need = pam_hip_gemm_workspace_bytes(1, m, n, k);
+    if (need > kScratchBytes)
+        return pamhost::fail(PAM_HIP_ERR_WORKSPACE, "pam_matmul_fwd_noalloc: this shape needs %zu bytes of scratch, the library holds %zu; "
+                             "use pam_hip_pam_matmul_fwd with a workspace", need, kScratchBytes);
+    void* ws = nullptr;
+    if (need > 0) {
+        const int rc = scratch_address("pam_matmul_fwd_noalloc", &ws);
+        if (rc != PAM_HIP_OK) return rc;
+    }
+    return gemm("pam_matmul_fwd_noalloc", MODE_PAM, 1, m, n, k, a, 0, a_sr, a_sc, b, 0, b_sr, b_sc, nullptr, 0, 0, 0,
+                y, 0, y_sr, y_sc, offset, ws, need, stream);
 }
 
 int pam_hip_pam_linear_fwd(const float* a, long a_sr, long a_sc, const float* b, long b_sr, long b_sc, const float* bias,
