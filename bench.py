@@ -57,8 +57,8 @@ def main():
     from pam_amd import _abi
     from pam_amd._abi import HipKernels
     from pam_amd import build as hip_build
-    if not hip_build.LIB.exists():            # the built library travels with the tree; build only when there is none
-        hip_build.build()
+    # the built library travels with the tree; it is rebuilt only if it is missing or was built from other sources
+    _, source_stamp = hip_build.ensure_built()
     _abi.load_library()
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")

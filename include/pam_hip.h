@@ -41,18 +41,12 @@ enum {
 
 int pam_hip_abi_version(void);
 const char *pam_hip_last_error(void);
+/* Hash of the sources and flags this library was built from (pam_amd/build.py writes it in), so that a test
+ * run or a benchmark can tell that the binary it loaded belongs to the tree it sits in. */
+const char *pam_hip_source_hash(void);
 
 /* Compute units and shader clock (kHz) of the current device, for roofline figures. */
 int pam_hip_device_info(int *compute_units, int *clock_khz);
-
-/* Measurement aid, no counterpart in the reference: runs the matrix kernel's instruction mix (one v_add_u32
- * and one dependent v_add_f32 per product) on register operands only, blocks work-groups of 256 lanes, each lane
- * iters * 256 VALU lane-operations; timing it gives the vector issue rate the roofline figures are stated against.
- * seed: 1024 words, out: blocks * 256 floats. */
-int pam_hip_issue_probe(const void *seed, float *out, int blocks, int iters, void *stream);
-/* The same with every step's operands read from LDS as the matrix kernel's inner loop reads them, for a
- * tm x tn micro-tile (4x4, 8x4, 8x8); each lane iters * 32 * tm * tn pairs. */
-int pam_hip_issue_probe_lds(const void *seed, float *out, int blocks, int iters, int tm, int tn, void *stream);
 
 /* ---- elementwise, n contiguous elements (pam/cuda_kernels.cu:141-328) ------------------ */
 /* C = A (*) B                         replaces pam_fwd  (elementwise_pam_caller,  :155-183) */
@@ -81,6 +75,9 @@ int pam_hip_pam_fwd_bcast(const float *x, const float *s, int scalar_is_a, float
 int pam_hip_pad_fwd_bcast(const float *x, const float *s, int scalar_is_a, float *c, size_t n, float offset, void *stream);
 
 /* ---- piecewise-affine exp / log (pam/cuda_kernels.cu:334-516) -------------------------- */
+/* The fp32 constant log2(base) that the four entry points below use: the double-precision logarithm rounded once
+ * (the reference's kernel evaluates log2(base) per element on the device, :343, 385, 438, 481). */
+float pam_hip_log2_base(float base);
 /* Y = base^X  = pa_exp2(X (*) log2 base)        replaces pa_exp_fwd (:348-373) */
 int pam_hip_pa_exp_fwd(const float *x, float *y, size_t n, float base, float offset, void *stream);
 /*                                                replaces pa_exp_bwd (:395-423) */
@@ -89,11 +86,6 @@ int pam_hip_pa_exp_bwd(const float *x, const float *dy, float *dx, size_t n, flo
 int pam_hip_pa_log_fwd(const float *x, float *y, size_t n, float base, float offset, void *stream);
 /*                                                replaces pa_log_bwd (:488-516) */
 int pam_hip_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, float base, float offset, void *stream);
-
-/* Tuning hook for experiments: forces the k-tile depth (16 or 32; 0 = automatic) and the number of
- * k chunks (0 = automatic) of the matrix products for the calling process.  No counterpart in the
- * reference; pam_hip_gemm_plan and pam_hip_gemm_workspace_bytes follow the forced values. */
-void pam_hip_set_tuning(int k_tile, int k_chunks);
 
 /* ---- matrix products (pam/cuda_kernels.cu:574-927) ------------------------------------- */
 /* A matrix operand: pointer, batch stride, row stride, column stride (elements). */

@@ -131,6 +131,18 @@ def pad_bwd(a, b, delta, offset=None):
     return _ternary("pamo_pad_bwd", a, b, delta, offset)
 
 
+def pad_grads_native(a, b, delta, offset=None, flavour="chain"):
+    """(dA, dB) of C = A (/) B as the reference's CPU autograd function computes them with approx_bwd=True
+    (pam/native.py:173-188): dA = pad(delta, B) without the offset, dB = -pad(pam(A, delta), pam(B, B)), each of
+    those three with the offset.  The GPU path of the reference, which this repository's kernels follow, uses other
+    formulas (pam/cuda_bindings.py:78-97); PAM is not associative, so the two differ in the last bits.
+    flavour "chain" models the float emulation of native.py bit for bit, "exact" is the integer definition."""
+    mul, div = (pam_chain, pad_chain) if flavour == "chain" else (pam, pad)
+    d_a = div(delta, b)
+    d_b = -div(mul(a, delta, offset), mul(b, b, offset), offset)
+    return d_a, d_b
+
+
 def pa_log2_raw(x):
     x = _f32(x); y = np.empty_like(x)
     lib().pamo_pa_log2(_p(x), _p(y), x.size)

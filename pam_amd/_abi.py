@@ -24,6 +24,7 @@ _MAT2 = [_p, _l, _l]             # pointer, row stride, col stride
 _SIGNATURES = {
     "pam_hip_abi_version": ([], _i),
     "pam_hip_last_error": ([], ctypes.c_char_p),
+    "pam_hip_source_hash": ([], ctypes.c_char_p),
     "pam_hip_device_info": ([ctypes.POINTER(_i), ctypes.POINTER(_i)], _i),
     "pam_hip_pam_fwd": ([_p, _p, _p, _z, _f, _p], _i),
     "pam_hip_pam_bwd": ([_p, _p, _p, _p, _z, _f, _p], _i),
@@ -31,6 +32,7 @@ _SIGNATURES = {
     "pam_hip_pad_bwd": ([_p, _p, _p, _p, _z, _f, _p], _i),
     "pam_hip_pam_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
     "pam_hip_pad_fwd_bcast": ([_p, _p, _i, _p, _z, _f, _p], _i),
+    "pam_hip_log2_base": ([_f], _f),
     "pam_hip_pa_exp_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_exp_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
     "pam_hip_issue_probe": ([_p, _p, _i, _i, _p], _i),

@@ -49,7 +49,10 @@
 #include <cstring>
 #include <mutex>
 
+#include <atomic>
+
 #include "pam_common.h"
+#include "../../include/pam_hip_probe.h"
 #include "pam_device.h"
 
 using namespace pamdev;
@@ -61,6 +64,9 @@ enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3 };   // k conti
 
 constexpr int KGRAN = 32;         // k ranges handed to work-groups are multiples of this
 constexpr int PAD = 4;
+// gfx950 parts (MI350X, MI355X) have eight XCDs, each with its own L2, and work-groups are dealt to them in turn.
+// The unit mapping built on this is a bijection for any count, so only locality depends on it.
+constexpr int XCDS = 8;
 
 struct Operand { const float* p; long sb, sr, sk; };    // batch, row (the non-k index), k strides
 
@@ -81,7 +87,7 @@ struct GemmArgs {
     int M, N, K;
     int ksplit, kchunk;          // kchunk is a multiple of 32; ksplit == 1 means no split
     int tiles, batch;            // output tiles per matrix, matrices
-    long xcd_chunk, units;       // xcd_chunk > 0: a 1-D launch, work-group x takes unit (x % 8) * xcd_chunk + x / 8 (see the launch)
+    long xcd_chunk, units;       // xcd_chunk > 0: a 1-D launch, work-group x takes unit (x % XCDS) * xcd_chunk + x / XCDS (see the launch)
     float off; int has_off;      // has_off: 0 none, 1 a normal number (off_add = its bit-pattern increment), 2 any other value
     uint32_t off_add;
 };
@@ -364,7 +370,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     const int ntn = (g.N + BN - 1) / BN;                  // consecutive tiles share L rows
     int tile = blockIdx.x, zs = blockIdx.y, zb = blockIdx.z;
     if (g.xcd_chunk > 0) {                                // units (matrix, k chunk, tile), one contiguous range per XCD
-        const long unit = (long)(blockIdx.x % 8) * g.xcd_chunk + (long)(blockIdx.x / 8);
+        const long unit = (long)(blockIdx.x % XCDS) * g.xcd_chunk + (long)(blockIdx.x / XCDS);
         if (unit >= g.units) return;                      // the ranges are rounded up: a few work-groups have nothing to do
         tile = (int)(unit % g.tiles);
         const long rest = unit / g.tiles;
@@ -714,23 +720,27 @@ __global__ __launch_bounds__(256) void splitk_reduce_vec_kernel(const v4f* __res
     y[idx] = total;
 }
 
-int g_cus = 0;
+// compute units of the current device (looked up once per device)
 int cu_count()
 {
-    if (g_cus == 0) {
-        int dev = 0; hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
-            g_cus = prop.multiProcessorCount;
-        else
-            g_cus = 256;
+    constexpr int kDevices = 64;
+    static std::atomic<int> cus[kDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kDevices) return 256;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        hipDeviceProp_t prop;
+        n = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+        cus[dev].store(n, std::memory_order_relaxed);
     }
-    return g_cus;
+    return n;
 }
 
 struct Plan { int bk; int ksplit; int kchunk; };
 
-// Tuning override for experiments: bk 0 = automatic (16 or 32), ksplit 0 = automatic.
-int g_force_bk = 0, g_force_ksplit = 0;
+// Tuning override for experiments, per calling thread (include/pam_hip_probe.h): bk 0 = automatic (16 or 32),
+// ksplit 0 = automatic.
+thread_local int g_force_bk = 0, g_force_ksplit = 0;
 
 // Work-groups own 64 x 64 output tiles.  k of 128 and more in whole multiples of 32, and any k
 // from 512, uses 32-deep k-tiles (fewer barriers and more bytes in flight per round, measured 3-5 %
@@ -808,8 +818,8 @@ void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& 
     // (not for few tiles with many k chunks, the weight-gradient shape: measured 8 % slower that way)
     if (units >= 64 && units < (1L << 31) - 8 && (p.ksplit == 1 || (long)grid.x >= cu_count())) {
         ga.units = units;
-        ga.xcd_chunk = (units + 7) / 8;
-        grid = dim3((unsigned)(8 * ga.xcd_chunk), 1, 1);
+        ga.xcd_chunk = (units + XCDS - 1) / XCDS;
+        grid = dim3((unsigned)(XCDS * ga.xcd_chunk), 1, 1);
     }
     if (p.bk == 32) launch_kinds<32, MODE>(lk, rk, grid, st, ga, partial);
     else launch_kinds<16, MODE>(lk, rk, grid, st, ga, partial);

@@ -65,3 +65,26 @@ def mixed_operands(n, seed, edge_frac=0.02):
                   [np.uint32(0), sub, np.uint32(0x7f800000), np.uint32(0x7fc00000), big, sub >> np.uint32(9)])
     x[idx] = f32((u.astype(np.uint32) | sign).astype(np.uint32))
     return x
+
+
+def ulp_histogram(got, want):
+    """{distance in units of the last place: count} between two fp32 arrays of finite values, as a JSON-ready dict."""
+    g = np.ascontiguousarray(np.asarray(got, dtype=np.float32)).view(np.int32).astype(np.int64)
+    w = np.ascontiguousarray(np.asarray(want, dtype=np.float32)).view(np.int32).astype(np.int64)
+    dist, count = np.unique(np.abs(g - w), return_counts=True)
+    return {str(int(d)): int(c) for d, c in zip(dist, count)}
+
+
+def full_mantissa_histograms(fns):
+    """The histograms kept in tests/golden/ulp_histogram.json: for each of pam, pad with and without the offset, the
+    distance between `fns[op](a, b, offset)` and what pam/native.py gave on the same operands (normal_fullmant.npz),
+    separately for its N(0,1) half and its wide-exponent half (|e| up to 40)."""
+    g = np.load(GOLDEN / "normal_fullmant.npz")
+    a, b = f32(g["a"]), f32(g["b"]); off = float(g["offset"]); n = a.size
+    out = {}
+    for name in ("pam", "pad", "pam_off", "pad_off"):
+        got = fns[name.split("_")[0]](a, b, off if name.endswith("_off") else None)
+        want = f32(g[name])
+        out[name] = {"unit_normal": ulp_histogram(got[:n // 2], want[:n // 2]),
+                     "wide_exponent": ulp_histogram(got[n // 2:], want[n // 2:])}
+    return out

@@ -14,12 +14,13 @@ def pytest_configure(config):
 
 @pytest.fixture(scope="session", autouse=True)
 def built_library():
-    """The tests load the library that is built; only when none is there do they build it (hipcc cross-compiles
-    without a GPU).  The package itself never builds or falls back: without the library it raises."""
+    """The tests load the library that is built, provided it was built from this tree's sources (it carries their
+    hash); a missing or stale one is rebuilt first (hipcc cross-compiles without a GPU).  The package itself never
+    builds or falls back: without the library it raises."""
     from pam_amd import build as builder
-    if not builder.LIB.exists():
-        builder.build()
-    return builder.LIB
+    lib, stamp = builder.ensure_built()
+    print(f"libpam_hip.so built from sources {stamp}")
+    return lib
 
 
 @pytest.fixture(scope="session")

@@ -8,6 +8,7 @@ pam/cuda_bindings.py:19-25.  Only inputs and outputs are stored, as uint32 bit
 patterns, so that signed zeros and NaNs survive.
 
     python tests/golden/make_goldens.py            # writes tests/golden/*.npz
+    python tests/golden/make_goldens.py pad_bwd    # only the file(s) of the named section(s)
 
 Functions covered are those that nothing but running the reference can pin: the
 output bits of native.pam_fwd / pad_fwd on full-mantissa inputs, the edge-class grid,
@@ -57,6 +58,9 @@ def main():
     torch.manual_seed(0)
     torch.set_num_threads(8)
     OFF = 1.0552
+    only = set(sys.argv[1:])
+    if only == {"pad_bwd"}:
+        return pad_bwd_section(native, OFF)
 
     # ---- 1. edge-class grid: all pairs of edge values
     ev = edge_values()
@@ -162,6 +166,8 @@ def main():
     print(f"native.pam_matmul config 0: fwd {t1 - t0:.3f} s, approx bwd {t2 - t1:.3f} s, "
           f"{torch.get_num_threads()} threads")
 
+    pad_bwd_section(native, OFF)
+
     # ---- timing of the elementwise reference path (for the baseline table)
     for n_log in (24,):
         n = 1 << n_log
@@ -173,6 +179,23 @@ def main():
                 t0 = time.perf_counter(); fn(A, B); ts.append(time.perf_counter() - t0)
             t = sorted(ts)[1]
             print(f"native.{name} n=2^{n_log}: {t:.3f} s  ({12 * n / t / 1e9:.3f} GB/s at 12 B/elem)")
+
+
+def pad_bwd_section(native, OFF):
+    """native.pad with approx_bwd=True through torch autograd (pam/native.py:173-196): the CPU flavour of the
+    quotient's gradients, which differs from the GPU flavour of pam/cuda_bindings.py:78-97."""
+    g = torch.Generator().manual_seed(4)
+    n = 4096
+    A = torch.randn(n, generator=g); B = torch.randn(n, generator=g); D = torch.randn(n, generator=g)
+    A[n // 2:] *= 2.0 ** torch.randint(-20, 20, (n // 2,), generator=g).float()
+    B[n // 2:] *= 2.0 ** torch.randint(-20, 20, (n // 2,), generator=g).float()
+    d = {"a": u32(A), "b": u32(B), "d": u32(D), "offset": np.float32(OFF)}
+    for tag, off in (("", None), ("_off", OFF)):
+        a = A.clone().requires_grad_(); b = B.clone().requires_grad_()
+        c = native.pad(a, b, offset=off, approx_bwd=True)
+        c.backward(D)
+        d["c" + tag] = u32(c); d["da" + tag] = u32(a.grad); d["db" + tag] = u32(b.grad)
+    np.savez_compressed(OUT / "pad_native_bwd.npz", **d)
 
 
 if __name__ == "__main__":

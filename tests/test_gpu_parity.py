@@ -139,6 +139,11 @@ def test_goldens_full_mantissa(K, oracle):
         assert same_bits(chain(a, b, o), want)[differ].all(), name
     assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), 1.0)), f32(g["pam_bwd"]), "pam_bwd")
     assert_same_bits(host(K.pam_bwd(dev(a), dev(b), dev(d), off)), f32(g["pam_bwd_off"]), "pam_bwd offset")
+    # how far the kernels are from pam/native.py, per unit of the last place: the recorded histogram
+    import json
+    from _util import full_mantissa_histograms
+    fns = {"pam": lambda x, y, o: host(K.pam_fwd(dev(x), dev(y), _o(o))), "pad": lambda x, y, o: host(K.pad_fwd(dev(x), dev(y), _o(o)))}
+    assert full_mantissa_histograms(fns) == json.loads((GOLDEN / "ulp_histogram.json").read_text())
 
 
 def test_goldens_edge_grid_classes(K):
@@ -285,6 +290,25 @@ def test_bmm_tails_and_strides(K, oracle):
     assert q.stride() == (Dh, BH * Dh, 1) and kt.stride() == (Dh, 1, BH * Dh)
     want = ogemm(oracle, np.swapaxes(x, 0, 1), np.swapaxes(np.swapaxes(y, 0, 1), 1, 2))
     assert_same_bits(host(K.pam_bmm_fwd(q, kt, True, False, 1.0)), want, "strided batch")
+    # the ordinary-multiply products through the batched kernel instances (pam/cuda_kernels.cu:942): every layout,
+    # the strided batch, and the autograd wrapper with BMM=True against torch.bmm on exactly representable products
+    want = ogemm(oracle, Q, Kt, mode=oracle.MODE_STD)
+    for ll, tl in _layouts(Q).items():
+        for lr, tr in _layouts(Kt).items():
+            assert_same_bits(host(K.standard_bmm(tl, tr, True, True, 1.0)), want, f"standard bmm {ll} x {lr}")
+    want = ogemm(oracle, np.swapaxes(x, 0, 1), np.swapaxes(np.swapaxes(y, 0, 1), 1, 2), mode=oracle.MODE_STD)
+    assert_same_bits(host(K.standard_bmm(q, kt, True, False, 1.0)), want, "standard bmm, strided batch")
+    from pam_amd import cuda_bindings
+    rng = np.random.RandomState(16)
+    a = dev((rng.randint(-8, 9, (5, 33, 20)) / 4.0).astype(np.float32)).requires_grad_()
+    b = dev((2.0 ** rng.randint(-3, 4, (5, 20, 17))).astype(np.float32)).requires_grad_()
+    up = dev((2.0 ** rng.randint(-2, 3, (5, 33, 17))).astype(np.float32))
+    out = cuda_bindings.standard_matmul(a, b, BMM=True)
+    out.backward(up)
+    a2, b2 = a.detach().clone().requires_grad_(), b.detach().clone().requires_grad_()
+    ref = torch.bmm(a2, b2)
+    ref.backward(up)
+    assert torch.equal(out, ref) and torch.equal(a.grad, a2.grad) and torch.equal(b.grad, b2.grad)
 
 
 def test_split_k_fixed_order(K, oracle):
@@ -333,6 +357,15 @@ def test_deit_linear_full_size(K, oracle):
     assert_same_bits(host(dX)[rows], ogemm(oracle, dY[rows], W, plan_shape=(1, 12608, 192, 768)), "dX rows")
     cols = rng.choice(768, 24, replace=False)
     assert_same_bits(host(dW)[:, cols], ogemm(oracle, X.T, dY[:, cols], plan_shape=(1, 192, 768, 12608)), "dW cols")
+    # the second layer of the pair, 768 -> 192: row-major times column-major with k = 768 (k split across work-groups)
+    X2 = rng.standard_normal((12608, 768)).astype(np.float32)
+    W2 = np.clip(rng.standard_normal((192, 768)) * 0.02, -0.04, 0.04).astype(np.float32)
+    Y2 = K.pam_matmul_fwd(dev(X2), dev(W2).T, True, False, 1.0)
+    assert_same_bits(host(Y2)[rows], ogemm(oracle, X2[rows], W2.T, plan_shape=(1, 12608, 192, 768)), "Y rows, 768 -> 192")
+    dY2 = (rng.standard_normal((12608, 192)) * 1e-2).astype(np.float32)
+    dW2 = K.pam_matmul_fwd(dev(X2).T, dev(dY2), False, True, 1.0)
+    cols2 = rng.choice(192, 16, replace=False)
+    assert_same_bits(host(dW2)[:, cols2], ogemm(oracle, X2.T, dY2[:, cols2], plan_shape=(1, 768, 192, 12608)), "dW cols, 768 -> 192")
     # multiplying an operand by a power of two multiplies every PAM product, hence the sum, exactly
     assert torch.equal(K.pam_matmul_fwd(tX * 4.0, tW.T, True, False, 1.0), Y * 4.0)
     assert torch.equal(K.pam_matmul_fwd(tX, (tW * 0.5).T, True, False, 1.0), Y * 0.5)

@@ -21,7 +21,11 @@ ROOT = pathlib.Path(__file__).resolve().parent.parent
 def test_library_exports_every_declared_symbol():
     header = (ROOT / "include" / "pam_hip.h").read_text()
     declared = set(re.findall(r"\b(pam_hip_[a-z0-9_]+)\s*\(", header))
-    assert len(declared) == 43
+    assert len(declared) == 42
+    # measurement probes and the tuning hook live in a header of their own, not in the drop-in interface
+    probes = set(re.findall(r"\b(pam_hip_[a-z0-9_]+)\s*\(", (ROOT / "include" / "pam_hip_probe.h").read_text()))
+    assert probes == {"pam_hip_issue_probe", "pam_hip_issue_probe_lds", "pam_hip_set_tuning"} and not (probes & declared)
+    declared |= probes
     lib = ctypes.CDLL(str(_abi.library_path()))
     missing = [name for name in sorted(declared) if not hasattr(lib, name)]
     assert not missing, f"declared in pam_hip.h but not exported: {missing}"
@@ -31,6 +35,22 @@ def test_library_exports_every_declared_symbol():
         assert "pam_hip_" + name in declared and hasattr(_abi.HipKernels, name)
     assert set(_abi.exported_symbols()) <= declared
     assert _abi.load_library().pam_hip_abi_version() == 1
+    # the library under test was built from the sources of this tree
+    from pam_amd import build as builder
+    assert _abi.load_library().pam_hip_source_hash().decode() == builder.source_hash()
+
+
+def test_log2_of_the_usual_bases_is_pinned():
+    """pa_exp / pa_log scale by the fp32 constant log2(base); one unit of the last place in it moves every result.
+    The goldens of tests/golden/exp_log.npz were written with torch.log2(torch.tensor(base)) on the CPU: the
+    library's constant, the oracle's and torch's must be these bit patterns."""
+    import numpy as np
+    import torch
+    from oracle import pam_oracle
+    lib = _abi.load_library()
+    for base, want in ((math.e, 0x3fb8aa3b), (10.0, 0x40549a78), (0.5, 0xbf800000), (2.0, 0x3f800000), (3.0, 0x3fcae00d)):
+        for got in (lib.pam_hip_log2_base(base), pam_oracle.log2_base(base), torch.log2(torch.tensor(base, dtype=torch.float32)).item()):
+            assert np.float32(got).view(np.uint32) == want, (base, got)
 
 
 def test_argument_errors_come_back_as_status_codes():

@@ -89,6 +89,43 @@ def test_full_mantissa(oracle):
         assert 0.1 < (ulp == 0).mean() < 0.6       # native.py is NOT the integer add on general inputs
 
 
+def test_ulp_histogram_is_the_recorded_one(oracle):
+    """Distance between the integer definition and pam/native.py per ulp, the kept artifact
+    tests/golden/ulp_histogram.json (tests/golden/make_ulp_histogram.py writes it)."""
+    import json
+    from _util import full_mantissa_histograms
+    kept = json.loads((GOLDEN / "ulp_histogram.json").read_text())
+    assert full_mantissa_histograms({"pam": oracle.pam, "pad": oracle.pad}) == kept
+    for name, halves in kept.items():
+        unit = halves["unit_normal"]; total = sum(unit.values())
+        assert unit["0"] / total > 0.6 and max(map(int, unit)) <= 16, name            # N(0,1): two thirds identical, the rest a few ulp
+        assert max(map(int, halves["wide_exponent"])) <= 96, name                     # |e| up to 40 costs native.py ~6 bits
+
+
+def test_quotient_gradients_of_the_cpu_flavour(oracle):
+    """pam/native.py:173-188 (pad_autograd, approx_bwd=True) computes the quotient's gradients by other formulas
+    than pam/cuda_bindings.py:78-97, which the kernels follow.  The oracle keeps native's as an alternate:
+    its chain flavour equals what torch autograd gave through native.pad bit for bit, its exact flavour to the
+    reference's tolerance, and the two flavours of gradient agree to PAM's own accuracy."""
+    g = np.load(GOLDEN / "pad_native_bwd.npz")
+    a, b, d = f32(g["a"]), f32(g["b"]), f32(g["d"]); off = float(g["offset"])
+    assert not (below_pow2(a) | below_pow2(b) | below_pow2(d)).any()
+    for tag, o in (("", None), ("_off", off)):
+        assert_same_bits(oracle.pad_chain(a, b, o), f32(g["c" + tag]), "forward" + tag)
+        da, db = oracle.pad_grads_native(a, b, d, o, flavour="chain")
+        keep = ~(below_pow2(oracle.pam_chain(a, d, o)) | below_pow2(oracle.pam_chain(b, b, o)))    # intermediate values in the log2 band
+        assert_same_bits(da, f32(g["da" + tag]), "dA" + tag)
+        assert_same_bits(db[keep], f32(g["db" + tag])[keep], "dB" + tag)
+        assert keep.mean() > 0.999
+        ea, eb = oracle.pad_grads_native(a, b, d, o, flavour="exact")
+        assert np.allclose(ea, f32(g["da" + tag]), rtol=1e-5, atol=1e-12) and np.allclose(eb[keep], f32(g["db" + tag])[keep], rtol=1e-5, atol=1e-12)
+        # the GPU flavour (pam/cuda_bindings.py:78-97): dA = pam(pad(1, B), delta), dB = -pam(pad(pad(A, B), B), delta)
+        one = np.ones_like(a)
+        ga = oracle.pam(oracle.pad(one, b, o), d, o)
+        gb = -oracle.pam(oracle.pad(oracle.pad(a, b, o), b, o), d, o)
+        assert np.allclose(ga, ea, rtol=0.15) and np.allclose(gb, eb, rtol=0.25)      # each PAM op is within 1/9 of the true one
+
+
 def test_pow2_band(oracle):
     g = np.load(GOLDEN / "pow2_band.npz")
     x = f32(g["x"]); glitch = below_pow2(x)
