@@ -91,8 +91,31 @@ __device__ __forceinline__ float pad_from_split(const Split& a, const Split& b)
     return u2f(join_mag(sign, eb - 127, frac));
 }
 
+// Any class of operands, without a branch: the hardware's frexp takes subnormal operands apart, the two fractions are
+// added exactly in fp32 (23-bit fractions, sums below 2), and ldexp puts the result together with the one rounding
+// that gradual underflow needs (nearest even) and the overflow to inf.  What remains are selects: results at or below
+// 2^-150 are zero (the reference evaluates 2**E first, pam/native.py:38-39), a zero operand gives a zero with the
+// sign of the other operand only, an inf or NaN operand gives NaN.
+//   |a| = ma 2^xa with ma in [0.5, 1): fraction fa = 2 ma - 1, exponent xa - 1; ga = ma - 0.5 = fa / 2.
+constexpr unsigned kClassZero = 0x060u;     // v_cmp_class masks: 0x060 = +-0, 0x207 = signalling NaN, quiet NaN, -inf, +inf
+
 __device__ __forceinline__ float pam_general(uint32_t ai, uint32_t bi)
-{ return pam_from_split(split_operand(ai, 127), split_operand(bi, 0)); }
+{
+    const float a = u2f(ai), b = u2f(bi);
+    const float ga = __builtin_amdgcn_frexp_mantf(__builtin_fabsf(a)) - 0.5f, gb = __builtin_amdgcn_frexp_mantf(__builtin_fabsf(b)) - 0.5f;
+    const int xa = __builtin_amdgcn_frexp_expf(a), xb = __builtin_amdgcn_frexp_expf(b);
+    const float s = ga + gb;                                   // (fa + fb) / 2, exact
+    const bool carry = s >= 0.5f;
+    const float half_mant = carry ? s : s + 0.5f;               // (fa + fb) / 2 or (1 + fa + fb) / 2, in [0.5, 1), exact
+    const int e2 = xa + xb + (carry ? 0 : -1);                  // result = half_mant 2^e2, its exponent E = e2 - 1
+    float r = __builtin_amdgcn_ldexpf(half_mant, e2);
+    r = e2 <= -149 ? 0.0f : r;
+    const bool za = __builtin_amdgcn_classf(a, kClassZero), zb = __builtin_amdgcn_classf(b, kClassZero);
+    const uint32_t sign = ((za ? 0u : ai) ^ (zb ? 0u : bi)) & kSign;
+    uint32_t out = (za | zb) ? sign : (f2u(r) | sign);
+    const bool bad = __builtin_amdgcn_classf(a, 0x207u) | __builtin_amdgcn_classf(b, 0x207u);    // NaN or inf
+    return u2f(bad ? kQNaN : out);
+}
 
 // PAM product a (*) b.
 __device__ __forceinline__ float pam_mul(float a, float b)
@@ -106,8 +129,26 @@ __device__ __forceinline__ float pam_mul(float a, float b)
     return pam_general(ai, bi);
 }
 
+// The quotient the same way: the fractions are subtracted; a negative difference borrows from the exponent.
+// x / +-0 is +-inf by the sign of x, 0 / 0 is NaN, 0 / y is a zero with the sign of y only, inf or NaN anywhere is NaN
+// (pam/native.py:163-164).
 __device__ __forceinline__ float pad_general(uint32_t ai, uint32_t bi)
-{ return pad_from_split(split_operand(ai, 127), split_operand(bi, 0)); }
+{
+    const float a = u2f(ai), b = u2f(bi);
+    const float ga = __builtin_amdgcn_frexp_mantf(__builtin_fabsf(a)), gb = __builtin_amdgcn_frexp_mantf(__builtin_fabsf(b));
+    const int xa = __builtin_amdgcn_frexp_expf(a), xb = __builtin_amdgcn_frexp_expf(b);
+    const float d = ga - gb;                                    // (fa - fb) / 2, exact, in (-0.5, 0.5)
+    const bool borrow = d < 0.0f;
+    const float half_mant = borrow ? d + 1.0f : d + 0.5f;        // (2 + fa - fb) / 2 or (1 + fa - fb) / 2, in [0.5, 1), exact
+    const int e2 = xa - xb + (borrow ? 0 : 1);                   // result = half_mant 2^e2
+    float r = __builtin_amdgcn_ldexpf(half_mant, e2);
+    r = e2 <= -149 ? 0.0f : r;
+    const bool za = __builtin_amdgcn_classf(a, kClassZero), zb = __builtin_amdgcn_classf(b, kClassZero);
+    const uint32_t sign = ((za ? 0u : ai) ^ (zb ? 0u : bi)) & kSign;
+    uint32_t out = zb ? ((ai & kSign) | kExpo) : za ? sign : (f2u(r) | sign);
+    const bool bad = __builtin_amdgcn_classf(a, 0x207u) | __builtin_amdgcn_classf(b, 0x207u) | (za & zb);
+    return u2f(bad ? kQNaN : out);
+}
 
 // PAM quotient a (/) b.
 __device__ __forceinline__ float pad_div(float a, float b)
