@@ -347,11 +347,9 @@ __device__ __forceinline__ void pam_mac_4x4(float (&acc)[4][4], const u32x4& a, 
 #undef PAM_MAC_ROW
 }
 
-#ifdef PAM_GEMM_WAVES
-#define PAM_GEMM_OCCUPANCY __attribute__((amdgpu_waves_per_eu(PAM_GEMM_WAVES)))
-#else
-#define PAM_GEMM_OCCUPANCY
-#endif
+// Four work-groups per compute unit are what the LDS allows; the register budget follows (128 per lane), so that no
+// instance of the kernel falls to three wavefronts per SIMD.
+#define PAM_GEMM_OCCUPANCY __attribute__((amdgpu_waves_per_eu(4)))
 
 template <int BM, int BN, int TM, int TN, int BK, int MODE, int LKIND, int RKIND>
 __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm_kernel(GemmArgs g, float* __restrict__ partial)
@@ -587,20 +585,34 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                 pam_mac_4x4(acc, fa[kk & 1], fb[kk & 1], pl, pr);
             }
         } else {
-            uint32_t fa[2][TM], fb[2][TN];
-            fragment(0, fa[0], fb[0]);
+            // The other modes leave the instructions to the compiler but keep the k-steps apart: an empty asm
+            // statement that the LDS addresses and the accumulators pass through, so that the reads of the step
+            // after next cannot move above this step's products (all of them at the top cost 300 registers).
+            static_assert(TM == 4 && TN == 4, "the step fence names sixteen accumulators");
+            typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
+            uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            u32x4 va[2], vb[2];
+            va[0] = *reinterpret_cast<LdsVec>(pl); vb[0] = *reinterpret_cast<LdsVec>(pr);
 #pragma unroll
             for (int kk = 0; kk < BK; ++kk) {
-                if (kk + 1 < BK) fragment(kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+                if (kk + 1 < BK) {
+                    va[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
+                    vb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
+                }
+                const uint32_t fa[4] = {va[kk & 1].x, va[kk & 1].y, va[kk & 1].z, va[kk & 1].w};
+                const uint32_t fb[4] = {vb[kk & 1].x, vb[kk & 1].y, vb[kk & 1].z, vb[kk & 1].w};
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) {
-                        if (MODE == MODE_PAM) acc[i][j] += u2f(fa[kk & 1][i] + fb[kk & 1][j]);
-                        else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f(fb[kk & 1][j]), acc[i][j]);
-                        else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(fa[kk & 1][i]), u2f((fb[kk & 1][j] + dfrac[i][j]) & ~kMant), acc[i][j]);
-                        else acc[i][j] = fmaf(u2f(fb[kk & 1][j]), u2f((fa[kk & 1][i] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                        if (MODE == MODE_PAM) acc[i][j] += u2f(fa[i] + fb[j]);
+                        else if (MODE == MODE_STD) acc[i][j] = fmaf(u2f(fa[i]), u2f(fb[j]), acc[i][j]);
+                        else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(fa[i]), u2f((fb[j] + dfrac[i][j]) & ~kMant), acc[i][j]);
+                        else acc[i][j] = fmaf(u2f(fb[j]), u2f((fa[i] + dfrac[i][j]) & ~kMant), acc[i][j]);
                     }
+                asm volatile("" : "+v"(pl), "+v"(pr),
+                             "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]),
+                             "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3]), "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3]));
             }
         }
     };
