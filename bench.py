@@ -48,6 +48,29 @@ def event_time_ms(fn, iters, torch):
     return start.elapsed_time(stop) / iters
 
 
+def config1_operand(n, seed, torch, dev):
+    """An operand of benchmark configuration 1: 98 % N(0,1); 2 % edge values at seeded random places, drawn uniformly
+    from +0, -0, subnormals of either sign with a random 23-bit mantissa, +-inf, NaN, and +-[FLT_MAX / 8, FLT_MAX]."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(n, generator=g)
+    k = n // 50
+    idx = torch.randperm(n, generator=g)[:k]
+    kind = torch.randint(0, 6, (k,), generator=g)
+    sign = torch.randint(0, 2, (k,), generator=g).to(torch.int64) << 31
+    mant = torch.randint(1, 1 << 23, (k,), generator=g).to(torch.int64)
+    big = 0x7f7fffff - torch.randint(0, 3 << 23, (k,), generator=g).to(torch.int64)
+    bits = torch.zeros(k, dtype=torch.int64)                                     # kind 0: +0, kind 1: -0 (sign forced below)
+    bits = torch.where(kind == 2, mant, bits)                                    # subnormal
+    bits = torch.where(kind == 3, torch.full_like(bits, 0x7f800000), bits)       # inf
+    bits = torch.where(kind == 4, torch.full_like(bits, 0x7fc00000), bits)       # NaN
+    bits = torch.where(kind == 5, big, bits)                                     # near FLT_MAX
+    sign = torch.where(kind == 0, torch.zeros_like(sign), torch.where(kind == 1, torch.full_like(sign, 1 << 31), sign))
+    u = (bits | sign)
+    u = torch.where(u >= (1 << 31), u - (1 << 32), u).to(torch.int32)
+    x[idx] = u.view(torch.float32)
+    return x.to(dev)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -150,16 +173,12 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "DeiT-tiny PAM linear fwd+dX+dW, tokens 64x197=12608, 192->768 and 768->192 "
                                "(benchmark configuration 2); 6 products of 1 859 125 248 PAM-MAC per step"},
-        "roofline": roofline, "products": per,
+        "roofline": roofline, "products": per, "library_source_hash": source_stamp,
     }
 
     if not args.no_elementwise:
         n = 1 << 26
-        a = torch.randn(n, generator=g).to(dev); b = torch.randn(n, generator=g).to(dev)
-        idx = torch.randint(0, n, (n // 50,), generator=g).to(dev)         # 2 % edge values
-        edge = torch.tensor([0.0, -0.0, float("inf"), float("nan"), 1e-40, -1e-41, 3e38, -2.5e38], device=dev)
-        a[idx] = edge[torch.arange(idx.numel(), device=dev) % 8]
-        b[idx.flip(0)] = edge[(torch.arange(idx.numel(), device=dev) + 3) % 8]
+        a = config1_operand(n, 10, torch, dev); b = config1_operand(n, 11, torch, dev)
         ew = {}
         for name, fn in (("mul", lambda: K.pam_fwd(a, b, 1.0)), ("div", lambda: K.pad_fwd(a, b, 1.0))):
             ms = event_time_ms(fn, 20, torch)
