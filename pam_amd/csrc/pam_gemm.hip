@@ -347,6 +347,40 @@ __device__ __forceinline__ void pam_mac_4x4(float (&acc)[4][4], const u32x4& a, 
 #undef PAM_MAC_ROW
 }
 
+// The exact-backward products of a 4 x 4 micro-tile for one k (pam/cuda_kernels.cu:48-57): per product the slope
+// operand's bits plus the kept fraction, masked to sign and exponent, times the upstream gradient, added by one
+// fma.  DELTA_LEFT: the gradient is the left fragment (a) and the slope operand the right one (b); else the reverse.
+// Two statements of eight products; the LDS addresses pass through as in pam_mac_4x4.
+template <bool DELTA_LEFT>
+__device__ __forceinline__ void pam_bwd_mac_4x4(float (&acc)[4][4], const uint32_t (&dfrac)[4][4], const u32x4& a, const u32x4& b,
+                                                uint32_t& pl, uint32_t& pr)
+{
+    uint32_t t0, t1;
+    if (DELTA_LEFT) {
+    asm volatile("v_add_u32 %[t0], %[b0], %[d00]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d01]\nv_fma_f32 %[c00], %[a0], %[t0], %[c00]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d02]\nv_fma_f32 %[c01], %[a0], %[t1], %[c01]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d03]\nv_fma_f32 %[c02], %[a0], %[t0], %[c02]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b0], %[d10]\nv_fma_f32 %[c03], %[a0], %[t1], %[c03]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d11]\nv_fma_f32 %[c10], %[a1], %[t0], %[c10]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d12]\nv_fma_f32 %[c11], %[a1], %[t1], %[c11]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d13]\nv_fma_f32 %[c12], %[a1], %[t0], %[c12]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c13], %[a1], %[t1], %[c13]\n"
+                     : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
+                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl)
+                     : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]),
+                       [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+        asm volatile("v_add_u32 %[t0], %[b0], %[d20]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d21]\nv_fma_f32 %[c20], %[a2], %[t0], %[c20]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d22]\nv_fma_f32 %[c21], %[a2], %[t1], %[c21]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d23]\nv_fma_f32 %[c22], %[a2], %[t0], %[c22]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b0], %[d30]\nv_fma_f32 %[c23], %[a2], %[t1], %[c23]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d31]\nv_fma_f32 %[c30], %[a3], %[t0], %[c30]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d32]\nv_fma_f32 %[c31], %[a3], %[t1], %[c31]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d33]\nv_fma_f32 %[c32], %[a3], %[t0], %[c32]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c33], %[a3], %[t1], %[c33]\n"
+                     : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
+                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr)
+                     : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]),
+                       [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+    } else {
+    asm volatile("v_add_u32 %[t0], %[a0], %[d00]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a0], %[d01]\nv_fma_f32 %[c00], %[b0], %[t0], %[c00]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a0], %[d02]\nv_fma_f32 %[c01], %[b1], %[t1], %[c01]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a0], %[d03]\nv_fma_f32 %[c02], %[b2], %[t0], %[c02]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a1], %[d10]\nv_fma_f32 %[c03], %[b3], %[t1], %[c03]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a1], %[d11]\nv_fma_f32 %[c10], %[b0], %[t0], %[c10]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a1], %[d12]\nv_fma_f32 %[c11], %[b1], %[t1], %[c11]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a1], %[d13]\nv_fma_f32 %[c12], %[b2], %[t0], %[c12]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c13], %[b3], %[t1], %[c13]\n"
+                     : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
+                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl)
+                     : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]),
+                       [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+        asm volatile("v_add_u32 %[t0], %[a2], %[d20]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a2], %[d21]\nv_fma_f32 %[c20], %[b0], %[t0], %[c20]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a2], %[d22]\nv_fma_f32 %[c21], %[b1], %[t1], %[c21]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a2], %[d23]\nv_fma_f32 %[c22], %[b2], %[t0], %[c22]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a3], %[d30]\nv_fma_f32 %[c23], %[b3], %[t1], %[c23]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a3], %[d31]\nv_fma_f32 %[c30], %[b0], %[t0], %[c30]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a3], %[d32]\nv_fma_f32 %[c31], %[b1], %[t1], %[c31]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a3], %[d33]\nv_fma_f32 %[c32], %[b2], %[t0], %[c32]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c33], %[b3], %[t1], %[c33]\n"
+                     : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
+                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr)
+                     : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]),
+                       [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+    }
+}
+
 // Four work-groups per compute unit are what the LDS allows; the register budget follows (128 per lane), so that no
 // instance of the kernel falls to three wavefronts per SIMD.
 #define PAM_GEMM_OCCUPANCY __attribute__((amdgpu_waves_per_eu(4)))
@@ -571,7 +605,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 
     // a full k-tile of in-range values: fragments for step kk+1 are read from LDS while step kk is computed
     auto plain_tile = [&]() {
-        if constexpr (MODE == MODE_PAM && TM == 4 && TN == 4) {
+        if constexpr (MODE != MODE_STD && TM == 4 && TN == 4) {
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
             u32x4 fa[2], fb[2];
@@ -582,7 +616,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                     fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
                     fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
                 }
-                pam_mac_4x4(acc, fa[kk & 1], fb[kk & 1], pl, pr);
+                if constexpr (MODE == MODE_PAM) pam_mac_4x4(acc, fa[kk & 1], fb[kk & 1], pl, pr);
+                else pam_bwd_mac_4x4<MODE == MODE_BWD_DL>(acc, dfrac, fa[kk & 1], fb[kk & 1], pl, pr);
             }
         } else {
             // The other modes leave the instructions to the compiler but keep the k-steps apart: an empty asm
