@@ -48,6 +48,7 @@
 #include <cmath>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 
 #include <atomic>
 
@@ -345,6 +346,56 @@ __device__ __forceinline__ void pam_mac_4x4(float (&acc)[4][4], const u32x4& a, 
           [t0] "=&v"(t0), [t1] "=&v"(t1), [pl] "+v"(pl), [pr] "+v"(pr)
         : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
 #undef PAM_MAC_ROW
+}
+
+// The same sixteen products for a k-tile whose LEFT (else right) operand holds zeros next to in-range values.  A PAM
+// product with a zero is +0 and adding it changes nothing (the sums start at +0 and never become -0), so those
+// products are not executed: per value of the operand with zeros one compare narrows the execution mask to the lanes
+// whose value is not the staged zero, the four products of that value run under it, and the mask is restored.  Two
+// instructions per product as in the plain block plus one compare per four products.
+template <bool LEFT>
+__device__ __forceinline__ void pam_mac_4x4_skip(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
+{
+    uint32_t t0, t1, t2, t3;
+    uint64_t all;
+    if (LEFT) {
+#define PAM_SKIP_ROW(I)                                                                         \
+    "v_cmpx_ne_u32_e32 vcc, 0, %[a" #I "]\n"                                                     \
+    "v_add_u32 %[t0], %[a" #I "], %[b0]\n v_add_u32 %[t1], %[a" #I "], %[b1]\n"                  \
+    "v_add_u32 %[t2], %[a" #I "], %[b2]\n v_add_u32 %[t3], %[a" #I "], %[b3]\n"                  \
+    "v_add_f32 %[c" #I "0], %[c" #I "0], %[t0]\n v_add_f32 %[c" #I "1], %[c" #I "1], %[t1]\n"    \
+    "v_add_f32 %[c" #I "2], %[c" #I "2], %[t2]\n v_add_f32 %[c" #I "3], %[c" #I "3], %[t3]\n"    \
+    "s_mov_b64 exec, %[all]\n"
+        asm volatile(
+            "s_mov_b64 %[all], exec\n" PAM_SKIP_ROW(0) PAM_SKIP_ROW(1) PAM_SKIP_ROW(2) PAM_SKIP_ROW(3)
+            : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),
+              [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
+              [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),
+              [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
+              [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [all] "=&s"(all), [pl] "+v"(pl), [pr] "+v"(pr)
+            : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w)
+            : "vcc");
+#undef PAM_SKIP_ROW
+    } else {
+#define PAM_SKIP_COL(J)                                                                         \
+    "v_cmpx_ne_u32_e32 vcc, %[zero], %[b" #J "]\n"                                               \
+    "v_add_u32 %[t0], %[a0], %[b" #J "]\n v_add_u32 %[t1], %[a1], %[b" #J "]\n"                  \
+    "v_add_u32 %[t2], %[a2], %[b" #J "]\n v_add_u32 %[t3], %[a3], %[b" #J "]\n"                  \
+    "v_add_f32 %[c0" #J "], %[c0" #J "], %[t0]\n v_add_f32 %[c1" #J "], %[c1" #J "], %[t1]\n"    \
+    "v_add_f32 %[c2" #J "], %[c2" #J "], %[t2]\n v_add_f32 %[c3" #J "], %[c3" #J "], %[t3]\n"    \
+    "s_mov_b64 exec, %[all]\n"
+        asm volatile(
+            "s_mov_b64 %[all], exec\n" PAM_SKIP_COL(0) PAM_SKIP_COL(1) PAM_SKIP_COL(2) PAM_SKIP_COL(3)
+            : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),
+              [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
+              [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),
+              [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
+              [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [all] "=&s"(all), [pl] "+v"(pl), [pr] "+v"(pr)
+            : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w),
+              [zero] "s"(kZeroR)
+            : "vcc");
+#undef PAM_SKIP_COL
+    }
 }
 
 // The exact-backward products of a 4 x 4 micro-tile for one k (pam/cuda_kernels.cu:48-57): per product the slope
@@ -652,6 +703,25 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         }
     };
 
+    // a full k-tile with zeros in one operand: the plain tile's schedule around the blocks that skip the zero products
+    auto skip_tile = [&](auto left) __attribute__((always_inline)) {
+        if constexpr (MODE == MODE_PAM && TM == 4 && TN == 4) {
+            typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
+            uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            u32x4 fa[2], fb[2];
+            fa[0] = *reinterpret_cast<LdsVec>(pl); fb[0] = *reinterpret_cast<LdsVec>(pr);
+#pragma unroll
+            for (int kk = 0; kk < BK; ++kk) {
+                if (kk + 1 < BK) {
+                    fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
+                    fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
+                }
+                pam_mac_4x4_skip<decltype(left)::value>(acc, fa[kk & 1], fb[kk & 1], pl, pr);
+            }
+        }
+    };
+    constexpr bool kSkips = MODE == MODE_PAM && TM == 4 && TN == 4;
+
     int t = 0;
     while (t < ktiles) {
         begin_tile(t);
@@ -664,6 +734,13 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             begin_tile(t);
         }
         if (t == ktiles) break;
+        // full k-tiles with zeros in one operand (activations after a ReLU)
+        if (kSkips && kcount == BK && (verdict == kZerosL || verdict == kZerosR)) {
+            if (verdict == kZerosL) skip_tile(std::true_type()); else skip_tile(std::false_type());
+            end_tile(t);
+            ++t;
+            continue;
+        }
         if (verdict == 0) {
 #pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) fast_step(kk);
