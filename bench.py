@@ -228,6 +228,9 @@ def main():
         X2r = torch.relu(X2)
         exact["fwd_12608x192x768_relu_input"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2r, W2.T, True, False, 1.0))
         exact["dW_768x192x12608_relu_input"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2r.T, dY2, False, True, 1.0))
+        # zeros in both operands: the same input against a weight matrix with 30 % of its entries pruned
+        W2s = W2 * (torch.rand(W2.shape, generator=g) >= 0.3).to(dev)
+        exact["fwd_12608x192x768_relu_input_pruned_weight"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2r, W2s.T, True, False, 1.0))
         for name, (ops, macs, fn) in exact.items():
             ms = event_time_ms(fn, 30, torch)
             other[name] = {"ms": round(ms, 4), "gmacs": round(macs / ms / 1e6, 1), "valu_frac": round(ops * macs / (ms * 1e-3) / lane_peak, 4)}

@@ -398,6 +398,41 @@ __device__ __forceinline__ void pam_mac_4x4_skip(float (&acc)[4][4], const u32x4
     }
 }
 
+// Zeros in both operands: a product runs in the lanes where neither value is the staged zero.  Eight compares give
+// the masks of the four left and four right values, the integer sums of a row are formed in all lanes, and each
+// float add runs under the AND of its two masks (formed on the scalar unit).
+__device__ __forceinline__ void pam_mac_4x4_skip_both(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
+{
+    uint32_t t0, t1, t2, t3;
+    uint64_t all, ma0, ma1, ma2, ma3, mb0, mb1, mb2, mb3;
+#define PAM_BOTH_ROW(I)                                                                         \
+    "s_mov_b64 exec, %[all]\n"                                                                  \
+    "v_add_u32 %[t0], %[a" #I "], %[b0]\n v_add_u32 %[t1], %[a" #I "], %[b1]\n"                  \
+    "v_add_u32 %[t2], %[a" #I "], %[b2]\n v_add_u32 %[t3], %[a" #I "], %[b3]\n"                  \
+    "s_and_b64 exec, %[ma" #I "], %[mb0]\n v_add_f32 %[c" #I "0], %[c" #I "0], %[t0]\n"          \
+    "s_and_b64 exec, %[ma" #I "], %[mb1]\n v_add_f32 %[c" #I "1], %[c" #I "1], %[t1]\n"          \
+    "s_and_b64 exec, %[ma" #I "], %[mb2]\n v_add_f32 %[c" #I "2], %[c" #I "2], %[t2]\n"          \
+    "s_and_b64 exec, %[ma" #I "], %[mb3]\n v_add_f32 %[c" #I "3], %[c" #I "3], %[t3]\n"
+    asm volatile(
+        "s_mov_b64 %[all], exec\n"
+        "v_cmp_ne_u32_e64 %[ma0], 0, %[a0]\n v_cmp_ne_u32_e64 %[ma1], 0, %[a1]\n"
+        "v_cmp_ne_u32_e64 %[ma2], 0, %[a2]\n v_cmp_ne_u32_e64 %[ma3], 0, %[a3]\n"
+        "v_cmp_ne_u32_e64 %[mb0], %[zero], %[b0]\n v_cmp_ne_u32_e64 %[mb1], %[zero], %[b1]\n"
+        "v_cmp_ne_u32_e64 %[mb2], %[zero], %[b2]\n v_cmp_ne_u32_e64 %[mb3], %[zero], %[b3]\n"
+        PAM_BOTH_ROW(0) PAM_BOTH_ROW(1) PAM_BOTH_ROW(2) PAM_BOTH_ROW(3)
+        "s_mov_b64 exec, %[all]\n"
+        : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),
+          [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
+          [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),
+          [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
+          [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [all] "=&s"(all),
+          [ma0] "=&s"(ma0), [ma1] "=&s"(ma1), [ma2] "=&s"(ma2), [ma3] "=&s"(ma3),
+          [mb0] "=&s"(mb0), [mb1] "=&s"(mb1), [mb2] "=&s"(mb2), [mb3] "=&s"(mb3), [pl] "+v"(pl), [pr] "+v"(pr)
+        : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w),
+          [zero] "s"(kZeroR));
+#undef PAM_BOTH_ROW
+}
+
 // The exact-backward products of a 4 x 4 micro-tile for one k (pam/cuda_kernels.cu:48-57): per product the slope
 // operand's bits plus the kept fraction, masked to sign and exponent, times the upstream gradient, added by one
 // fma.  DELTA_LEFT: the gradient is the left fragment (a) and the slope operand the right one (b); else the reverse.
@@ -703,8 +738,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         }
     };
 
-    // a full k-tile with zeros in one operand: the plain tile's schedule around the blocks that skip the zero products
-    auto skip_tile = [&](auto left) __attribute__((always_inline)) {
+    // a full k-tile with zeros: the plain tile's schedule around the blocks that skip the zero products
+    auto skip_tile = [&](auto which) __attribute__((always_inline)) {
         if constexpr (MODE == MODE_PAM && TM == 4 && TN == 4) {
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
@@ -716,7 +751,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                     fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
                     fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
                 }
-                pam_mac_4x4_skip<decltype(left)::value>(acc, fa[kk & 1], fb[kk & 1], pl, pr);
+                constexpr uint32_t kWhich = decltype(which)::value;
+                if constexpr (kWhich == (kZerosL | kZerosR)) pam_mac_4x4_skip_both(acc, fa[kk & 1], fb[kk & 1], pl, pr);
+                else pam_mac_4x4_skip<kWhich == kZerosL>(acc, fa[kk & 1], fb[kk & 1], pl, pr);
             }
         }
     };
@@ -734,9 +771,11 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             begin_tile(t);
         }
         if (t == ktiles) break;
-        // full k-tiles with zeros in one operand (activations after a ReLU)
-        if (kSkips && kcount == BK && (verdict == kZerosL || verdict == kZerosR)) {
-            if (verdict == kZerosL) skip_tile(std::true_type()); else skip_tile(std::false_type());
+        // full k-tiles with zeros (activations after a ReLU, padding, pruned weights)
+        if (kSkips && kcount == BK && verdict != 0 && verdict < kGuarded) {
+            if (verdict == kZerosL) skip_tile(std::integral_constant<uint32_t, kZerosL>());
+            else if (verdict == kZerosR) skip_tile(std::integral_constant<uint32_t, kZerosR>());
+            else skip_tile(std::integral_constant<uint32_t, kZerosL | kZerosR>());
             end_tile(t);
             ++t;
             continue;
