@@ -417,9 +417,34 @@ void pamo_gemm_fast(long M, long N, long K, const float *L, const float *R, floa
  * softmax gradient as autograd chains the primitives' backward formulas
  * (pam/cuda_bindings.py:43-57, 78-97, 224-239).  The one thing the reference leaves open,
  * the order of torch.sum along a row, is fixed to the order of the GPU kernels:
- * 64 strided partial sums from +0, then a butterfly p[l] = p[l] + p[l ^ s], s = 32 .. 1. */
+ * 64 strided partial sums from +0, then a butterfly p[l] = p[l] + p[l ^ s], s = 32 .. 1.
+ * Rows of 4097 ... 16384 values are summed by 1024 threads instead: 1024 strided partial sums
+ * from +0, the butterfly within each group of 64 consecutive partial sums, then the 16 group
+ * sums added in ascending order. */
+static float butterfly64(const float *in)
+{
+    float p[64], q[64];
+    memcpy(p, in, sizeof p);
+    for (int s = 32; s >= 1; s >>= 1) {
+        for (int l = 0; l < 64; ++l) { volatile float t = p[l] + p[l ^ s]; q[l] = t; }
+        memcpy(p, q, sizeof p);
+    }
+    return p[0];
+}
+
 static float row_sum_fixed(const float *v, long n)
 {
+    if (n > 4096 && n <= 16384) {
+        float part[1024];
+        for (int t = 0; t < 1024; ++t) {
+            volatile float s = 0.0f;
+            for (long i = t; i < n; i += 1024) s = s + v[i];
+            part[t] = s;
+        }
+        volatile float total = butterfly64(part);
+        for (int w = 1; w < 16; ++w) total = total + butterfly64(part + 64 * w);
+        return total;
+    }
     float p[64], q[64];
     for (int l = 0; l < 64; ++l) {
         volatile float s = 0.0f;

@@ -15,6 +15,8 @@
 // maximum sweep, 4 in, 4 out), 12 for its backward, 8 for layer_norm and log_softmax.
 #include <math.h>
 
+#include <atomic>
+
 #include "pam_common.h"
 #include "pam_device.h"
 
@@ -47,6 +49,40 @@ __device__ __forceinline__ float wave_sum(float p)
     for (int s = 32; s >= 1; s >>= 1) p = p + __shfl_xor(p, s, 64);
     return p;
 }
+
+// Who holds which element of a row and how partial sums over the row are combined.
+// WaveRow: one wavefront per row, lane l holds the elements l, l + 64, ...
+// BlockRow: a work-group of 1024 threads per row (rows of 4097 ... 16384 values), thread t holds t, t + 1024, ...;
+// its sums: every wavefront folds its 64 partial sums by the butterfly, then the 16 wavefront sums are added in
+// ascending order, ((w0 + w1) + w2) + ... + w15, by every thread itself.  Two slots of LDS alternate, so one
+// barrier per sum is enough (a thread can be at most one sum ahead of the slowest).
+constexpr int kBlockThreads = 1024, kBlockWaves = kBlockThreads / 64;
+constexpr long kBlockRowMin = 4096, kBlockRowMax = 16L * kBlockThreads;       // the block kernels take kBlockRowMin < n <= kBlockRowMax
+struct WaveRow {
+    static constexpr int kStride = 64;
+    int id;
+    __device__ __forceinline__ long index(int c) const { return id + 64L * c; }
+    __device__ __forceinline__ float sum(float p) { return wave_sum(p); }
+    __device__ __forceinline__ bool all(bool ok) { return __ballot(!ok) == 0ull; }
+};
+struct BlockRow {
+    static constexpr int kStride = kBlockThreads;
+    int id; float (*slots)[kBlockWaves]; int turn;
+    __device__ __forceinline__ long index(int c) const { return id + (long)kBlockThreads * c; }
+    __device__ __forceinline__ float sum(float p)
+    {
+        p = wave_sum(p);
+        float* slot = slots[turn];
+        turn ^= 1;
+        if (id % 64 == 0) slot[id / 64] = p;
+        __syncthreads();
+        float t = slot[0];
+#pragma unroll
+        for (int w = 1; w < kBlockWaves; ++w) t = t + slot[w];
+        return t;
+    }
+    __device__ __forceinline__ bool all(bool ok) { return __syncthreads_and(ok ? 1 : 0) != 0; }
+};
 
 // maximum that propagates NaN, as torch.max does
 struct MaxNan {
@@ -129,6 +165,18 @@ __device__ __forceinline__ void load_row(float (&v)[CH], const float* __restrict
 #pragma unroll
     for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; v[c] = i < n ? p[i] : fill; }
 }
+template <int CH, class L>
+__device__ __forceinline__ void load_row(float (&v)[CH], const float* __restrict__ p, long n, const L& lay, float fill)
+{
+#pragma unroll
+    for (int c = 0; c < CH; ++c) { const long i = lay.index(c); v[c] = i < n ? p[i] : fill; }
+}
+template <int CH, class L>
+__device__ __forceinline__ void store_row(const float (&v)[CH], float* __restrict__ p, long n, const L& lay)
+{
+#pragma unroll
+    for (int c = 0; c < CH; ++c) { const long i = lay.index(c); if (i < n) p[i] = v[c]; }
+}
 
 // p = p + f(x[i]) over the lane's elements in ascending order
 template <class F>
@@ -181,8 +229,8 @@ __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
 }
 
 // one row held in registers: weights, their sum, the quotients; masked (-inf) elements weigh exactly zero
-template <int CH, class M>
-__device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)[CH], float shift, M& m)
+template <int CH, class M, class L>
+__device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)[CH], float shift, M& m, L& lay)
 {
     float p = 0.0f;
 #pragma unroll
@@ -193,7 +241,7 @@ __device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)
         out[c] = masked ? 0.0f : e;
         p = p + out[c];
     }
-    const float total = wave_sum(p);
+    const float total = lay.sum(p);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool masked = f2u(xv[c]) == 0xff800000u;
@@ -273,9 +321,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if constexpr (CH > 0) {
             float xv[CH], out[CH];
             load_row<CH>(xv, xr, n, lane, kNegInf);            // the fill has weight zero
+            WaveRow lay{lane};
             Unchecked u{o, Span()};
-            total = softmax_row<CH>(xv, out, shift, u);
-            if (!wave_valid(u)) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k); }
+            total = softmax_row<CH>(xv, out, shift, u, lay);
+            if (!wave_valid(u)) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k, lay); }
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
@@ -315,9 +364,9 @@ __device__ __forceinline__ float softmax_dx(float xv, float e, float g, float in
 // The all-approximate gradient of one register-resident row with unchecked arithmetic.  Masked
 // (-inf) elements and the lanes past the end of the row are computed on a stand-in value and
 // replaced by the zeros the chain gives them.
-template <int CH>
+template <int CH, class L>
 __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
-                                                        float total, float shift, int lane, long n, Unchecked& m)
+                                                        float total, float shift, L& lay, long n, Unchecked& m)
 {
     const float inv = m.div(1.0f, total);
     float e[CH];
@@ -325,7 +374,7 @@ __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], c
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool masked = f2u(xv[c]) == 0xff800000u;
-        const bool inside = lane + 64L * c < n;
+        const bool inside = lay.index(c) < n;
         const float t = m.mul(masked ? 1.0f : xv[c], kLog2E) - shift;
         e[c] = m.exp2(masked ? 0.5f : t);                                  // exp2 of the shifted input, unmasked
         // -(((e (/) total) (/) total) (*) g); a masked element has e = 0 and the checked chain gives
@@ -334,16 +383,33 @@ __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], c
         if (masked && inside) m.sp.see(f2u(g[c]) & ~kSign);
         if (inside && !masked) p = p + term;
     }
-    const float dtotal = wave_sum(p);
+    const float dtotal = lay.sum(p);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool masked = f2u(xv[c]) == 0xff800000u;
-        const bool inside = lane + 64L * c < n;
+        const bool inside = lay.index(c) < n;
         const float de = m.mul(inv, (inside && !masked) ? g[c] : 1.0f) + dtotal;
         const float dt = m.mul(m.mul(e[c], kLn2), de);
         const float dx = m.mul(dt, kLog2E);
         out[c] = masked ? 0.0f : dx;
     }
+}
+
+// The same gradient with the checked primitives, for every combination of exact and approximate terms.
+template <int CH, class L>
+__device__ __forceinline__ void softmax_grad_row_checked(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
+                                                         float total, float inv, float shift, L& lay, long n, Offset o, Approx ap)
+{
+    float e[CH];
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        e[c] = softmax_weight(xv[c], shift, o);
+        if (lay.index(c) < n) p = p + softmax_dsum_term(e[c], total, g[c], o, ap);
+    }
+    const float dtotal = lay.sum(p);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) out[c] = softmax_dx(xv[c], e[c], g[c], inv, dtotal, shift, o, ap);
 }
 
 template <int CH>
@@ -363,23 +429,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             load_row<CH>(xv, xr, n, lane, kNegInf);
             load_row<CH>(g, gr, n, lane, 0.0f);
             bool done = false;
+            WaveRow lay{lane};
             if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient has an unchecked form
                 Unchecked u{o, Span()};
-                softmax_grad_row_approx<CH>(xv, g, out, total, shift, lane, n, u);
+                softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
                 done = wave_valid(u);
             }
-            if (!done) {
-                float e[CH];
-                float p = 0.0f;
-#pragma unroll
-                for (int c = 0; c < CH; ++c) {
-                    e[c] = softmax_weight(xv[c], shift, o);
-                    if (lane + 64L * c < n) p = p + softmax_dsum_term(e[c], total, g[c], o, ap);
-                }
-                const float dtotal = wave_sum(p);
-#pragma unroll
-                for (int c = 0; c < CH; ++c) out[c] = softmax_dx(xv[c], e[c], g[c], inv, dtotal, shift, o, ap);
-            }
+            if (!done) softmax_grad_row_checked<CH>(xv, g, out, total, inv, shift, lay, n, o, ap);
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) dr[i] = out[c]; }
         } else {
@@ -419,18 +475,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 }
 
 // ---------------------------------------------------------------- logsumexp and log_softmax (pam/pam_ops.py:331-347)
-template <int CH, class M>
-__device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shift, int lane, long n, M& m)
+template <int CH, class M, class L>
+__device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shift, L& lay, long n, M& m)
 {
     float p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const bool inside = lane + 64L * c < n;                  // lanes past the end work on stand-in values
+        const bool inside = lay.index(c) < n;                    // lanes past the end work on stand-in values
         const float t = m.mul(inside ? xv[c] : 1.0f, kLog2E) - shift;
         const float e = m.exp2(inside ? t : 0.5f);
         if (inside) p = p + e;
     }
-    return m.div(shift + m.log2(wave_sum(p)), kLog2E);
+    return m.div(shift + m.log2(lay.sum(p)), kLog2E);
 }
 
 template <int CH>
@@ -447,9 +503,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if constexpr (CH > 0) {
             float xv[CH];
             load_row<CH>(xv, xr, n, lane, 0.0f);
+            WaveRow lay{lane};
             Unchecked u{o, Span()};
-            float out = logsumexp_row<CH>(xv, shift, lane, n, u);
-            if (!wave_valid(u)) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lane, n, k); }
+            float out = logsumexp_row<CH>(xv, shift, lay, n, u);
+            if (!wave_valid(u)) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lay, n, k); }
             if (lse && lane == 0) lse[r] = out;
             if (y) {
 #pragma unroll
@@ -487,25 +544,25 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restr
 }
 
 // ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
-template <int CH, class M>
+template <int CH, class M, class L>
 __device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&out)[CH], const float* __restrict__ weight,
-                                               const float* __restrict__ bias, int lane, long n, float count, float eps, M& m)
+                                               const float* __restrict__ bias, L& lay, long n, float count, float eps, M& m)
 {
     float p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) p = p + xv[c];                          // the fill adds +0
-    const float mu = m.div(wave_sum(p), count);
+    const float mu = m.div(lay.sum(p), count);
     p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         out[c] = xv[c] - mu;                                             // lanes past the end hold -mu, a stand-in
         const float sq = m.mul(out[c], out[c]);
-        if (lane + 64L * c < n) p = p + sq;
+        if (lay.index(c) < n) p = p + sq;
     }
-    const float denom = m.root(m.div(wave_sum(p), count) + eps);
+    const float denom = m.root(m.div(lay.sum(p), count) + eps);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const long i = lane + 64L * c; const bool inside = i < n;
+        const long i = lay.index(c); const bool inside = i < n;
         float r = m.div(out[c], denom);
         if (weight) r = m.mul(r, inside ? weight[i] : 1.0f);
         if (bias) r = r + (inside ? bias[i] : 0.0f);
@@ -526,9 +583,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if constexpr (CH > 0) {
             float xv[CH], out[CH];
             load_row<CH>(xv, xr, n, lane, 0.0f);
+            WaveRow lay{lane};
             Unchecked u{o, Span()};
-            layer_norm_row<CH>(xv, out, weight, bias, lane, n, count, eps, u);
-            if (!wave_valid(u)) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lane, n, count, eps, k); }
+            layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, u);
+            if (!wave_valid(u)) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, k); }
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
         } else {
@@ -601,27 +659,27 @@ struct GradUnchecked {
 // One row of the logsumexp / log_softmax gradient.  xv: the inputs (any fill past the end); gy: the
 // per-element gradients (log_softmax) with 1.0 past the end; out: dx.  Lanes past the end of the
 // row work on stand-in values that are never stored or summed.
-template <int CH, class G>
+template <int CH, class G, class L>
 __device__ __forceinline__ void logsumexp_grad_row(const float (&xv)[CH], const float (&gy)[CH], float (&out)[CH], float g_row,
-                                                   bool log_softmax, float shift, int lane, long n, G& m)
+                                                   bool log_softmax, float shift, L& lay, long n, G& m)
 {
     float p = 0.0f, q = 0.0f, t[CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const bool inside = lane + 64L * c < n;
+        const bool inside = lay.index(c) < n;
         const float s = m.mul(inside ? xv[c] : 1.0f, kLog2E) - shift;
         t[c] = inside ? s : 0.5f;
         const float e = m.exp2(t[c]);
         if (inside) { p = p + e; q = q + gy[c]; }
     }
-    const float total = wave_sum(p);
-    const float g_out = log_softmax ? -wave_sum(q) : g_row;         // x - lse: the broadcast lse collects -sum(gy)
+    const float total = lay.sum(p);
+    const float g_out = log_softmax ? -lay.sum(q) : g_row;         // log_softmax is the same for every thread of a launch         // x - lse: the broadcast lse collects -sum(gy)
     const float u = shift + m.log2(total);
     const float du = m.div_da(u, kLog2E, g_out);
     const float dtotal = m.log2_dx(total, du);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const bool inside = lane + 64L * c < n;
+        const bool inside = lay.index(c) < n;
         const float d = m.mul_da(inside ? xv[c] : 1.0f, kLog2E, m.exp2_dx(t[c], dtotal));
         out[c] = log_softmax ? gy[c] + d : d;
     }
@@ -644,12 +702,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         if (log_softmax) load_row<CH>(gy, grad + r * n, n, lane, 1.0f);
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
+        WaveRow lay{lane};
         if (ap.a && ap.b && ap.e) {
             GradUnchecked u{o, Span()};
-            logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lane, n, u);
+            logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
-        if (!done) { GradChecked k{o, ap}; logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lane, n, k); }
+        if (!done) { GradChecked k{o, ap}; logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, k); }
 #pragma unroll
         for (int c = 0; c < CH; ++c) { const long i = lane + 64L * c; if (i < n) dx[r * n + i] = out[c]; }
     }
@@ -726,19 +785,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 
 // One row of the layer_norm gradient.  cen: x on entry, overwritten; g: dy on entry (1.0 past the
 // end), dx on exit; terms: the per-element terms of the weight gradient (if weight).
-template <int CH, class G>
+template <int CH, class G, class L>
 __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)[CH], float (&terms)[CH],
-                                                    const float* __restrict__ weight, int lane, long n, float count, float eps, G& m)
+                                                    const float* __restrict__ weight, L& lay, long n, float count, float eps, G& m)
 {
     float p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) p = p + cen[c];                        // the fill adds +0
-    const float s1 = wave_sum(p);
+    const float s1 = lay.sum(p);
     const float mu = m.div(s1, count);
     p = 0.0f;
 #pragma unroll
-    for (int c = 0; c < CH; ++c) { cen[c] = cen[c] - mu; const float sq = m.mul(cen[c], cen[c]); if (lane + 64L * c < n) p = p + sq; }
-    const float s2 = wave_sum(p);
+    for (int c = 0; c < CH; ++c) { cen[c] = cen[c] - mu; const float sq = m.mul(cen[c], cen[c]); if (lay.index(c) < n) p = p + sq; }
+    const float s2 = lay.sum(p);
     const float v = m.div(s2, count) + eps;
     const float lg = m.log2(v);
     const float half = m.mul(lg, 0.5f);
@@ -748,7 +807,7 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
     p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const long i = lane + 64L * c; const bool inside = i < n;
+        const long i = lay.index(c); const bool inside = i < n;
         if (weight) {
             const float xn = m.div(cen[c], denom), wi = inside ? weight[i] : 1.0f;
             terms[c] = m.mul_db(xn, wi, g[c]);
@@ -757,7 +816,7 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
         const float d = m.div_db(cen[c], denom, g[c]);
         if (inside) p = p + d;
     }
-    float d = wave_sum(p);
+    float d = lay.sum(p);
     if (v == 0.0f) d = 0.0f;                                            // where(v == 0, 0, exp2(..))
     d = m.exp2_dx(half, d);
     d = m.mul_da(lg, 0.5f, d);
@@ -771,9 +830,9 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
         dc = dc + m.mul_da(cen[c], cen[c], ds2);
         dc = dc + m.mul_db(cen[c], cen[c], ds2);
         g[c] = dc;
-        if (lane + 64L * c < n) p = p + dc;
+        if (lay.index(c) < n) p = p + dc;
     }
-    const float ds1 = m.div_da(s1, count, -wave_sum(p));                // mu is subtracted: it collects -sum(dc)
+    const float ds1 = m.div_da(s1, count, -lay.sum(p));                // mu is subtracted: it collects -sum(dc)
 #pragma unroll
     for (int c = 0; c < CH; ++c) g[c] = g[c] + ds1;
 }
@@ -871,18 +930,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >
     for (long r = wave; r < rows; r += nwaves) {
         float cen[CH], g[CH], terms[CH];
         bool done = false;
+        WaveRow lay{lane};
         if (ap.a && ap.b && ap.e) {
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
             GradUnchecked u{o, Span()};
-            layer_norm_grad_row<CH>(cen, g, terms, weight, lane, n, count, eps, u);
+            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
         if (!done) {                                    // the row is read again (from cache) rather than kept in registers
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
             GradChecked k{o, ap};
-            layer_norm_grad_row<CH>(cen, g, terms, weight, lane, n, count, eps, k);
+            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, k);
         }
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
@@ -891,6 +951,199 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >
         }
     }
 }
+
+// ---------------------------------------------------------------- a work-group per row (rows of 4097 ... 16384 values)
+// One row is held in the registers of 1024 threads (CH values each), read once and written once; the row functions
+// are the ones above, with the work-group's sum in place of the wavefront's.  Whether the unchecked arithmetic
+// was valid is decided for the whole row, so that every thread takes the same path to the next barrier.
+#ifdef PAM_BLOCK_WAVES
+#define PAM_BLOCK_ATTR __attribute__((amdgpu_waves_per_eu(PAM_BLOCK_WAVES)))
+#else
+#define PAM_BLOCK_ATTR
+#endif
+// logsumexp forward, which needs the fewest registers: the input row of the next iteration is fetched while the
+// current one is computed (there is one work-group per compute unit, so nothing else would hide the latency;
+// the other kernels have no registers to spare for it).  Past the last row the fetch repeats the last row:
+// a conditional fetch would tie the registers to their old contents and make the compiler wait for them at once.
+#define PAM_BLOCK_FIRST_ROW(AHEAD, X, FILL) \
+    load_row<CH>(AHEAD, X + (blockIdx.x < rows ? (long)blockIdx.x : rows - 1) * n, n, lay, FILL)
+#define PAM_BLOCK_NEXT_ROW(NOW, AHEAD, X, FILL)                                                          \
+    _Pragma("unroll") for (int c = 0; c < CH; ++c) NOW[c] = AHEAD[c];                                    \
+    load_row<CH>(AHEAD, X + (r + gridDim.x < rows ? r + gridDim.x : rows - 1) * n, n, lay, FILL)
+#define PAM_BLOCK_ROW_SETUP                                                        \
+    __shared__ float red_slots[2][kBlockWaves];                                    \
+    BlockRow lay{(int)threadIdx.x, red_slots, 0};                                  \
+    const int lane = threadIdx.x % 64;                                             \
+    (void)lane
+
+template <int CH>
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_fwd_block_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                                         float* __restrict__ row_sum, float* __restrict__ shift_out,
+                                                                         long rows, long n, Offset o,
+                                                                         const float* __restrict__ partial, int partials)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float shift = fold_shift(partial, partials, lane);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        float xv[CH], out[CH];
+        load_row<CH>(xv, x + r * n, n, lay, kNegInf);
+        Unchecked u{o, Span()};
+        float total = softmax_row<CH>(xv, out, shift, u, lay);
+        if (!lay.all(u.valid())) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k, lay); }
+        store_row<CH>(out, y + r * n, n, lay);
+        if (threadIdx.x == 0) row_sum[r] = total;
+    }
+}
+
+template <int CH>
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_bwd_block_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                                         const float* __restrict__ row_sum, const float* __restrict__ shift_in,
+                                                                         float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float shift = *shift_in;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float total = row_sum[r];
+        float xv[CH], g[CH], out[CH];
+        load_row<CH>(xv, x + r * n, n, lay, kNegInf);
+        load_row<CH>(g, dy + r * n, n, lay, 0.0f);
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            Unchecked u{o, Span()};
+            softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
+            done = lay.all(u.valid());
+        }
+        if (!done) softmax_grad_row_checked<CH>(xv, g, out, total, pad_div_off(1.0f, total, o.off, o.has), shift, lay, n, o, ap);
+        store_row<CH>(out, dx + r * n, n, lay);
+    }
+}
+
+template <int CH>
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_block_kernel(const float* __restrict__ x, float* __restrict__ lse,
+                                                                       float* __restrict__ y, float* __restrict__ shift_out, long rows, long n,
+                                                                       Offset o, const float* __restrict__ partial, int partials)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float shift = fold_shift(partial, partials, lane);
+    if (shift_out && blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
+    float ahead[CH];
+    PAM_BLOCK_FIRST_ROW(ahead, x, 0.0f);
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        float xv[CH];
+        PAM_BLOCK_NEXT_ROW(xv, ahead, x, 0.0f);
+        Unchecked u{o, Span()};
+        float out = logsumexp_row<CH>(xv, shift, lay, n, u);
+        if (!lay.all(u.valid())) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lay, n, k); }
+        if (lse && threadIdx.x == 0) lse[r] = out;
+        if (y) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) { const long i = lay.index(c); if (i < n) y[r * n + i] = xv[c] - out; }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void row_mean_block_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                                      long rows, long n, Offset o)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float count = (float)n;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        const float* xr = x + r * n;
+        float p = 0.0f;
+#pragma unroll 4
+        for (long i = threadIdx.x; i < n; i += kBlockThreads) p = p + xr[i];
+        const float total = lay.sum(p);
+        if (threadIdx.x == 0) y[r] = pad_div_off(total, count, o.off, o.has);
+    }
+}
+
+template <int CH>
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_fwd_block_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                                                            const float* __restrict__ bias, float* __restrict__ y,
+                                                                            long rows, long n, float eps, Offset o)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float count = (float)n;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        float xv[CH], out[CH];
+        load_row<CH>(xv, x + r * n, n, lay, 0.0f);
+        Unchecked u{o, Span()};
+        layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, u);
+        if (!lay.all(u.valid())) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, k); }
+        store_row<CH>(out, y + r * n, n, lay);
+    }
+}
+
+template <int CH>
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_bwd_block_kernel(
+    const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
+    long rows, long n, int log_softmax, Offset o, Approx ap)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float shift = *shift_in;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        float xv[CH], gy[CH], out[CH];
+        load_row<CH>(xv, x + r * n, n, lay, 0.0f);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) gy[c] = 1.0f;
+        if (log_softmax) load_row<CH>(gy, grad + r * n, n, lay, 1.0f);
+        const float g_row = log_softmax ? 0.0f : grad[r];
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            GradUnchecked u{o, Span()};
+            logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, u);
+            done = lay.all(u.valid());
+        }
+        if (!done) { GradChecked k{o, ap}; logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, k); }
+        store_row<CH>(out, dx + r * n, n, lay);
+    }
+}
+
+template <int CH>
+__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_bwd_block_kernel(
+    const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
+    float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
+{
+    PAM_BLOCK_ROW_SETUP;
+    const float count = (float)n;
+    for (long r = blockIdx.x; r < rows; r += gridDim.x) {
+        float cen[CH], g[CH], terms[CH];
+        bool done = false;
+        if (ap.a && ap.b && ap.e) {
+            load_row<CH>(cen, x + r * n, n, lay, 0.0f);
+            load_row<CH>(g, gy + r * n, n, lay, 1.0f);
+            GradUnchecked u{o, Span()};
+            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, u);
+            done = lay.all(u.valid());
+        }
+        if (!done) {                                    // the row is read again (from cache) rather than kept in registers
+            load_row<CH>(cen, x + r * n, n, lay, 0.0f);
+            load_row<CH>(g, gy + r * n, n, lay, 1.0f);
+            GradChecked k{o, ap};
+            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, k);
+        }
+        store_row<CH>(g, dx + r * n, n, lay);
+        if (weight && dw_terms) store_row<CH>(terms, dw_terms + r * n, n, lay);
+    }
+}
+
+// values per thread of the block kernels for a row of n values
+int block_chunks(long n)
+{
+    for (int ch : {6, 8, 10, 12}) if (n <= (long)kBlockThreads * ch) return ch;
+    return 16;
+}
+bool block_rows(long n) { return n > kBlockRowMin && n <= kBlockRowMax; }
+
+#define PAM_BLOCK_DISPATCH(KERNEL, n, grid, st, ...)                                                            \
+    switch (block_chunks(n)) {                                                                                  \
+    case 6: hipLaunchKernelGGL(KERNEL<6>, grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;                \
+    case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;                \
+    case 10: hipLaunchKernelGGL(KERNEL<10>, grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;              \
+    case 12: hipLaunchKernelGGL(KERNEL<12>, grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;              \
+    default: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;              \
+    }
 
 // smallest register-resident variant that holds a row of n values, 0 for the streaming one
 int row_chunks(long n)
@@ -918,16 +1171,26 @@ int row_chunks(long n)
     default: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     }
 
-int g_cus = 0;
+// compute units of the current device (looked up once per device)
 int cu_count()
 {
-    if (g_cus == 0) {
-        int dev = 0; hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
-            g_cus = prop.multiProcessorCount;
-        else g_cus = 256;
+    static std::atomic<int> table[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int cus = table[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        cus = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+        table[dev].store(cus, std::memory_order_relaxed);
     }
-    return g_cus;
+    return cus;
+}
+
+// a work-group per row, at most four per compute unit in the launch
+unsigned block_grid(long rows)
+{
+    long cap = (long)cu_count() * 4;
+    return (unsigned)(rows < cap ? (rows < 1 ? 1 : rows) : cap);
 }
 
 // one wavefront per row, at most 16 wavefronts per SIMD's worth of work-groups in flight
@@ -977,8 +1240,13 @@ int pam_hip_softmax_fwd(const float* x, float* y, float* row_sum, float* shift, 
     hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
     rc = launch_max("softmax_fwd", x, rows, n, o, 1, workspace, workspace_bytes, st, &partials);
     if (rc != PAM_HIP_OK) return rc;
-    PAM_ROW_DISPATCH(softmax_fwd_kernel, n, dim3(row_grid(rows)), st, x, y, row_sum, shift, rows, n, o,
-                     (const float*)workspace, partials);
+    if (block_rows(n)) {
+        PAM_BLOCK_DISPATCH(softmax_fwd_block_kernel, n, dim3(block_grid(rows)), st, x, y, row_sum, shift, rows, n, o,
+                           (const float*)workspace, partials);
+    } else {
+        PAM_ROW_DISPATCH(softmax_fwd_kernel, n, dim3(row_grid(rows)), st, x, y, row_sum, shift, rows, n, o,
+                         (const float*)workspace, partials);
+    }
     return pamhost::check_launch("softmax_fwd");
 }
 
@@ -990,7 +1258,11 @@ int pam_hip_softmax_bwd(const float* x, const float* dy, const float* row_sum, c
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !dy || !row_sum || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "softmax_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    PAM_ROW_DISPATCH(softmax_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap);
+    if (block_rows(n)) {
+        PAM_BLOCK_DISPATCH(softmax_bwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap);
+    } else {
+        PAM_ROW_DISPATCH(softmax_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap);
+    }
     return pamhost::check_launch("softmax_bwd");
 }
 
@@ -1004,8 +1276,13 @@ int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, float*
     hipStream_t st = (hipStream_t)stream; Offset o{offset, offset != 1.0f}; int partials = 0;
     rc = launch_max("logsumexp_fwd", x, rows, n, o, 0, workspace, workspace_bytes, st, &partials);
     if (rc != PAM_HIP_OK) return rc;
-    PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows)), st, x, lse, log_softmax, shift, rows, n, o,
-                     (const float*)workspace, partials);
+    if (block_rows(n)) {
+        PAM_BLOCK_DISPATCH(logsumexp_block_kernel, n, dim3(block_grid(rows)), st, x, lse, log_softmax, shift, rows, n, o,
+                           (const float*)workspace, partials);
+    } else {
+        PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows)), st, x, lse, log_softmax, shift, rows, n, o,
+                         (const float*)workspace, partials);
+    }
     return pamhost::check_launch("logsumexp_fwd");
 }
 
@@ -1015,8 +1292,12 @@ int pam_hip_row_mean_fwd(const float* x, float* y, long rows, long n, float offs
     if (rc != PAM_HIP_OK) return rc;
     if (rows == 0) return PAM_HIP_OK;
     if (!y || (n > 0 && !x)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "row_mean_fwd: null pointer");
-    hipLaunchKernelGGL(row_mean_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, y, rows, n,
-                       Offset{offset, offset != 1.0f});
+    if (block_rows(n))
+        hipLaunchKernelGGL(row_mean_block_kernel, dim3(block_grid(rows)), dim3(kBlockThreads), 0, (hipStream_t)stream, x, y, rows, n,
+                           Offset{offset, offset != 1.0f});
+    else
+        hipLaunchKernelGGL(row_mean_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, y, rows, n,
+                           Offset{offset, offset != 1.0f});
     return pamhost::check_launch("row_mean_fwd");
 }
 
@@ -1028,7 +1309,11 @@ int pam_hip_layer_norm_fwd(const float* x, const float* weight, const float* bia
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !y) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_fwd: null pointer");
     const Offset o{offset, offset != 1.0f};
-    PAM_ROW_DISPATCH(layer_norm_fwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, bias, y, rows, n, eps, o);
+    if (block_rows(n)) {
+        PAM_BLOCK_DISPATCH(layer_norm_fwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, weight, bias, y, rows, n, eps, o);
+    } else {
+        PAM_ROW_DISPATCH(layer_norm_fwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, bias, y, rows, n, eps, o);
+    }
     return pamhost::check_launch("layer_norm_fwd");
 }
 
@@ -1040,7 +1325,10 @@ int pam_hip_logsumexp_bwd(const float* x, const float* grad, const float* shift,
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !grad || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    if (n > 1024)
+    if (block_rows(n)) {
+        PAM_BLOCK_DISPATCH(logsumexp_bwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n,
+                           log_softmax, o, ap);
+    } else if (n > 1024)
         hipLaunchKernelGGL(logsumexp_bwd_stream_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, grad, shift, dx,
                            rows, n, log_softmax, o, ap);
     else
@@ -1057,7 +1345,10 @@ int pam_hip_layer_norm_bwd(const float* x, const float* weight, const float* dy,
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !dy || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    if (n > 1024)
+    if (block_rows(n)) {
+        PAM_BLOCK_DISPATCH(layer_norm_bwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms,
+                           rows, n, eps, o, ap);
+    } else if (n > 1024)
         hipLaunchKernelGGL(layer_norm_bwd_stream_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, weight, dy, dx,
                            dw_terms, rows, n, eps, o, ap);
     else

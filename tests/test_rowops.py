@@ -25,9 +25,26 @@ OFF = 1.0552
 
 
 def fixed_sum(v):
-    """Row sums in the kernels' order: 64 strided partial sums from +0, then a butterfly."""
+    """Row sums in the kernels' order: 64 strided partial sums from +0, then a butterfly.  Rows of
+    4097 ... 16384 values: 1024 strided partial sums, the butterfly within each group of 64, then the
+    16 group sums in ascending order."""
     v = np.asarray(v, dtype=np.float32)
     rows, n = v.shape
+    if 4096 < n <= 16384:
+        pad = (-n) % 1024
+        if pad:
+            v = np.concatenate([v, np.zeros((rows, pad), np.float32)], axis=1)
+        p = np.zeros((rows, 1024), np.float32)
+        for j in range(v.shape[1] // 1024):
+            p = (p + v[:, 1024 * j:1024 * j + 1024]).astype(np.float32)
+        p = p.reshape(rows, 16, 64)
+        lanes = np.arange(64)
+        for s in (32, 16, 8, 4, 2, 1):
+            p = (p + p[:, :, lanes ^ s]).astype(np.float32)
+        total = p[:, 0, 0]
+        for w in range(1, 16):
+            total = (total + p[:, w, 0]).astype(np.float32)
+        return total
     pad = (-n) % 64
     if pad:
         v = np.concatenate([v, np.zeros((rows, pad), np.float32)], axis=1)     # adding +0 changes nothing
@@ -136,7 +153,7 @@ def test_oracle_softmax_special_rows(oracle):
 
 @pytest.mark.parametrize("off", [None, OFF])
 def test_oracle_logsumexp_mean_layer_norm_are_the_chains(oracle, off):
-    for rows, n in [(1, 1), (3, 7), (4, 64), (5, 192), (2, 513)]:
+    for rows, n in [(1, 1), (3, 7), (4, 64), (5, 192), (2, 513), (2, 4097), (2, 9000)]:
         x = rows_case(rows * 77 + n, rows, n, masks=False)
         want = logsumexp_chain(oracle, x, off)
         lse, ls = oracle.logsumexp_fwd(x, off, with_log_softmax=True)
@@ -236,7 +253,9 @@ def _dev(a):
 @pytest.mark.gpu
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_softmax_forward_backward(oracle, off):
-    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (64, 197), (2, 1000), (300, 32), (5, 4097)]:
+    # 4097 ... 16384 values: a work-group per row
+    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (64, 197), (2, 1000), (300, 32), (3, 4096), (5, 4097), (3, 6145), (2, 10000),
+                    (2, 16384), (2, 16385)]:
         x = rows_case(rows * 1000 + n, rows, n)
         g = np.random.RandomState(n).standard_normal(x.shape).astype(np.float32)
         want, row_sum, shift = oracle.softmax_fwd(x, off)
@@ -289,8 +308,42 @@ def test_gpu_softmax_special_values(oracle):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("off", [None, OFF])
+def test_gpu_long_rows_with_special_values(oracle, off):
+    """Rows held by a whole work-group: a value outside the normal range anywhere in the row sends every
+    thread of the row to the checked arithmetic (forward and all-approximate gradients)."""
+    n = 9000
+    x = rows_case(77, 6, n, masks=False)
+    x[1, 8999] = 0.0; x[2, 1024] = 1e-40; x[3, 5000] = np.inf; x[4, 63] = -np.inf; x[5, 4000] = np.nan
+    g = np.random.RandomState(8).standard_normal(x.shape).astype(np.float32)
+    g[0, 77] = 0.0; g[1, 5] = 1e-41
+    w = (np.random.RandomState(9).standard_normal(n) + 2).astype(np.float32); w[17] = 0.0
+    xt = _dev(x).requires_grad_()
+    y = pam_amd.softmax(xt, dim=-1, offset=off, approx_bwd=True)
+    want, row_sum, shift = oracle.softmax_fwd(x, off)
+    assert_same_bits(y.detach().cpu().numpy(), want, "softmax")
+    y.backward(_dev(g))
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, off, (True, True, True)), "softmax gradient")
+    xs = x[:3]                                       # finite rows for the shifted ops
+    lse, ls = oracle.logsumexp_fwd(xs, off, with_log_softmax=True)
+    xt = _dev(xs).requires_grad_()
+    y = pam_amd.log_softmax(xt, dim=-1, offset=off, approx_bwd=True)
+    assert_same_bits(y.detach().cpu().numpy(), ls, "log_softmax")
+    y.backward(_dev(g[:3]))
+    sh = np.floor(oracle.pam(xs, C, off).max())
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xs, g[:3], sh, off, (True, True, True), log_softmax=True), "log_softmax gradient")
+    assert_same_bits(pam_amd.mean(_dev(x), dim=-1, offset=off).cpu().numpy(), oracle.row_mean_fwd(x, off), "mean")
+    xt = _dev(x).requires_grad_(); wt = _dev(w).requires_grad_()
+    y = pam_amd.layer_norm(xt, n, wt, None, offset=off, approx_bwd=True)
+    assert_same_bits(y.detach().cpu().numpy(), oracle.layer_norm_fwd(x, w, None, 1e-5, off), "layer_norm")
+    y.backward(_dev(g))
+    dx, _ = oracle.layer_norm_bwd(x, w, g, 1e-5, off, (True, True, True))
+    assert_same_bits(xt.grad.cpu().numpy(), dx, "layer_norm gradient")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_logsumexp_mean_layer_norm(oracle, off):
-    for rows, n in [(1, 1), (3, 7), (4, 64), (50, 192), (2, 513), (33, 512), (3, 10000)]:
+    for rows, n in [(1, 1), (3, 7), (4, 64), (50, 192), (2, 513), (33, 512), (2, 4096), (3, 4097), (3, 8193), (3, 10000), (2, 12289), (2, 16384), (2, 16385)]:
         x = rows_case(rows * 77 + n, rows, n, masks=False)
         xt = _dev(x)
         lse, ls = oracle.logsumexp_fwd(x, off, with_log_softmax=True)
@@ -340,7 +393,7 @@ def test_gpu_attention_softmax_full_size(oracle):
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_logsumexp_and_layer_norm_gradients(oracle, off):
     # rows beyond 1024 values: the gradient kernels sweep the row several times instead of holding it in registers
-    for rows, n in [(1, 1), (3, 7), (5, 64), (40, 192), (9, 513), (6, 1024), (5, 1025), (3, 2500), (2, 10000)]:
+    for rows, n in [(1, 1), (3, 7), (5, 64), (40, 192), (9, 513), (6, 1024), (5, 1025), (3, 2500), (2, 4097), (2, 6200), (2, 10000), (2, 12300), (2, 16384), (2, 16385)]:
         x = rows_case(rows * 13 + n, rows, n, masks=False)
         rng = np.random.RandomState(n)
         g_rows = rng.standard_normal(rows).astype(np.float32); g_full = rng.standard_normal(x.shape).astype(np.float32)
