@@ -144,13 +144,22 @@ __global__ __launch_bounds__(kThreads) void scaled_max_kernel(const float* __res
     }
 }
 
-// every wavefront folds the per-block maxima itself (at most 4 KiB, cache resident): floor(max)
-__device__ __forceinline__ float fold_shift(const float* __restrict__ partial, int count, int lane)
+// The work-group folds the per-block maxima together (at most 4 KiB, cache resident), each wavefront a share of
+// them, and exchanges the results through LDS: floor(max).  The maximum does not depend on the order.
+template <int WAVES>
+__device__ __forceinline__ float fold_shift(const float* __restrict__ partial, int count)
 {
+    __shared__ float fold_mx[WAVES];
+    __shared__ int fold_nan[WAVES];
     MaxNan m;
-    for (int i = lane; i < count; i += 64) m.take(partial[i]);
+    for (int i = threadIdx.x; i < count; i += WAVES * 64) m.take(partial[i]);
     m.merge_wave();
-    return floorf(m.value());
+    if (threadIdx.x % 64 == 0) { fold_mx[threadIdx.x / 64] = m.mx; fold_nan[threadIdx.x / 64] = m.nan; }
+    __syncthreads();
+    MaxNan t;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) { t.mx = fmaxf(t.mx, fold_mx[w]); t.nan |= fold_nan[w] != 0; }
+    return floorf(t.value());
 }
 
 // ---------------------------------------------------------------- row access
@@ -313,7 +322,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
-    const float shift = fold_shift(partial, partials, lane);
+    const float shift = fold_shift<kWaves>(partial, partials);
     if (wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
@@ -496,7 +505,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
-    const float shift = fold_shift(partial, partials, lane);
+    const float shift = fold_shift<kWaves>(partial, partials);
     if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
@@ -983,7 +992,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_fwd_bloc
                                                                          const float* __restrict__ partial, int partials)
 {
     PAM_BLOCK_ROW_SETUP;
-    const float shift = fold_shift(partial, partials, lane);
+    const float shift = fold_shift<kBlockWaves>(partial, partials);
     if (blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float xv[CH], out[CH];
@@ -1025,7 +1034,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_block_
                                                                        Offset o, const float* __restrict__ partial, int partials)
 {
     PAM_BLOCK_ROW_SETUP;
-    const float shift = fold_shift(partial, partials, lane);
+    const float shift = fold_shift<kBlockWaves>(partial, partials);
     if (shift_out && blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     float ahead[CH];
     PAM_BLOCK_FIRST_ROW(ahead, x, 0.0f);
@@ -1193,11 +1202,13 @@ unsigned block_grid(long rows)
     return (unsigned)(rows < cap ? (rows < 1 ? 1 : rows) : cap);
 }
 
-// one wavefront per row, at most 16 wavefronts per SIMD's worth of work-groups in flight
-unsigned row_grid(long rows)
+// one wavefront per row, at most `per_cu` work-groups per compute unit in the launch: 16 (four wavefronts per SIMD's
+// worth of waiting work-groups) for most kernels, 8 (exactly what is resident) for the short-row forward kernels
+// that start by folding the shift, so that each wavefront does so once for more rows
+unsigned row_grid(long rows, int per_cu = 16)
 {
     long blocks = (rows + kWaves - 1) / kWaves;
-    long cap = (long)cu_count() * 16;
+    long cap = (long)cu_count() * per_cu;
     return (unsigned)(blocks < cap ? (blocks < 1 ? 1 : blocks) : cap);
 }
 
@@ -1244,7 +1255,7 @@ int pam_hip_softmax_fwd(const float* x, float* y, float* row_sum, float* shift, 
         PAM_BLOCK_DISPATCH(softmax_fwd_block_kernel, n, dim3(block_grid(rows)), st, x, y, row_sum, shift, rows, n, o,
                            (const float*)workspace, partials);
     } else {
-        PAM_ROW_DISPATCH(softmax_fwd_kernel, n, dim3(row_grid(rows)), st, x, y, row_sum, shift, rows, n, o,
+        PAM_ROW_DISPATCH(softmax_fwd_kernel, n, dim3(row_grid(rows, n <= 256 ? 8 : 16)), st, x, y, row_sum, shift, rows, n, o,
                          (const float*)workspace, partials);
     }
     return pamhost::check_launch("softmax_fwd");
@@ -1280,7 +1291,7 @@ int pam_hip_logsumexp_fwd(const float* x, float* lse, float* log_softmax, float*
         PAM_BLOCK_DISPATCH(logsumexp_block_kernel, n, dim3(block_grid(rows)), st, x, lse, log_softmax, shift, rows, n, o,
                            (const float*)workspace, partials);
     } else {
-        PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows)), st, x, lse, log_softmax, shift, rows, n, o,
+        PAM_ROW_DISPATCH(logsumexp_kernel, n, dim3(row_grid(rows, n <= 256 ? 8 : 16)), st, x, lse, log_softmax, shift, rows, n, o,
                          (const float*)workspace, partials);
     }
     return pamhost::check_launch("logsumexp_fwd");
