@@ -150,6 +150,10 @@ __device__ __forceinline__ uint32_t max3u(uint32_t a, uint32_t b, uint32_t c) { 
 // Verdict of a k-tile: bit 0 / bit 1 = the left / right operand holds zeros (all else in range),
 // kGuarded = some value needs the full definition.  Verdicts of wavefronts combine by OR.
 constexpr uint32_t kZerosL = 1u, kZerosR = 2u, kGuarded = 4u;
+// A wavefront all of whose rows lie beyond M (the last row tile of a matrix whose height is not a multiple of the
+// tile: 197 rows leave three of the four wavefronts of the fourth tile without a row) stages and synchronises with
+// the others but computes nothing.
+constexpr uint32_t kIdle = 8u;
 
 // Stand-ins that keep the integer sum a finite number when one operand is zero: 2^-64 on the
 // left, 2^64 (less the bias) on the right, just outside the range [2^-63, 2^64) that the other
@@ -567,6 +571,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     // per k-tile: where its fragments are in LDS, how many k it holds, and what the staging found in it
     const uint32_t* sl = nullptr; const uint32_t* sr = nullptr;
     int kcount = 0;
+    const bool idle_wave = MODE != MODE_STD && __builtin_amdgcn_readfirstlane(row0 + (wave * 64 / TXN) * 4 >= g.M ? 1 : 0) != 0;
     uint32_t verdict = 0;                         // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
     auto begin_tile = [&](int t) {
         const int cur = t & 1;
@@ -581,7 +586,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             uint32_t f = 0;
 #pragma unroll
             for (int w = 0; w < NW; ++w) f |= lds_flag[cur][w];
-            verdict = __builtin_amdgcn_readfirstlane(f);
+            verdict = idle_wave ? kIdle : __builtin_amdgcn_readfirstlane(f);
         }
         sl = lds_l[cur] + ty * 4;
         sr = lds_r[cur] + tx * 4;
@@ -771,6 +776,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             begin_tile(t);
         }
         if (t == ktiles) break;
+        if (verdict == kIdle) { end_tile(t); ++t; continue; }
         // full k-tiles with zeros (activations after a ReLU, padding, pruned weights)
         if (kSkips && kcount == BK && verdict != 0 && verdict < kGuarded) {
             if (verdict == kZerosL) skip_tile(std::integral_constant<uint32_t, kZerosL>());
