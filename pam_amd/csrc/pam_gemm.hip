@@ -530,7 +530,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     TileLoader<BM, NT, LKIND, BK> ll;
     TileLoader<BN, NT, RKIND, BK> rl;
 
-    auto stage = [&](int buf) {
+    auto stage = [&](int buf) __attribute__((always_inline)) {
         PlainStager<false> same{0u};
         if (MODE == MODE_STD) {
             ll.store(lds_l[buf], tid, same);
@@ -573,7 +573,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     int kcount = 0;
     const bool idle_wave = MODE != MODE_STD && __builtin_amdgcn_readfirstlane(row0 + (wave * 64 / TXN) * 4 >= g.M ? 1 : 0) != 0;
     uint32_t verdict = 0;                         // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
-    auto begin_tile = [&](int t) {
+    auto begin_tile = [&](int t) __attribute__((always_inline)) {
         const int cur = t & 1;
         const int k0 = kbegin + t * BK;
         // The next tile is fetched unconditionally: past the end the clamped addresses re-read the last
@@ -591,12 +591,12 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         sl = lds_l[cur] + ty * 4;
         sr = lds_r[cur] + tx * 4;
     };
-    auto end_tile = [&](int t) {
+    auto end_tile = [&](int t) __attribute__((always_inline)) {
         if (t + 1 < ktiles) stage((t & 1) ^ 1);
         __syncthreads();
     };
 
-    auto fragment = [&](int kk, uint32_t (&a)[TM], uint32_t (&b)[TN]) {
+    auto fragment = [&](int kk, uint32_t (&a)[TM], uint32_t (&b)[TN]) __attribute__((always_inline)) {
 #pragma unroll
         for (int gi = 0; gi < GM; ++gi) {
             uint4 q = *reinterpret_cast<const uint4*>(sl + kk * LDL + gi * (BM / GM));
@@ -608,7 +608,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             b[gj * 4 + 0] = q.x; b[gj * 4 + 1] = q.y; b[gj * 4 + 2] = q.z; b[gj * 4 + 3] = q.w;
         }
     };
-    auto fast_step = [&](int kk) {
+    auto fast_step = [&](int kk) __attribute__((always_inline)) {
         uint32_t a[TM], b[TN];
         fragment(kk, a, b);
 #pragma unroll
@@ -623,7 +623,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     };
     // k-tile with zeros but otherwise in range: the integer add of a zero is garbage, so those
     // products are replaced by +0 (one v_cndmask per product, masks combined on the scalar unit)
-    auto zeros_step = [&](int kk) {
+    auto zeros_step = [&](int kk) __attribute__((always_inline)) {
         uint32_t a[TM], b[TN];
         fragment(kk, a, b);
         bool za[TM], zb[TN];
@@ -640,7 +640,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     // the product is multiplied by 0 or 1 in the accumulating fma (x * 1 + acc rounds like acc + x;
     // x * 0 + acc leaves acc, which is never -0) -- two instructions per product like the plain loop,
     // plus three per value of the operand with zeros
-    auto zeros_left_step = [&](int kk) {
+    auto zeros_left_step = [&](int kk) __attribute__((always_inline)) {
         uint32_t a[TM], b[TN];
         fragment(kk, a, b);
         float keep[TM];
@@ -655,7 +655,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[i], acc[i][j]);
     };
-    auto zeros_right_step = [&](int kk) {
+    auto zeros_right_step = [&](int kk) __attribute__((always_inline)) {
         uint32_t a[TM], b[TN];
         fragment(kk, a, b);
         float keep[TN];
@@ -670,7 +670,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[j], acc[i][j]);
     };
-    auto guarded_step = [&](int kk) {
+    auto guarded_step = [&](int kk) __attribute__((always_inline)) {
         uint32_t a[TM], b[TN];
         fragment(kk, a, b);
         if (MODE == MODE_PAM) {
@@ -695,7 +695,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     };
 
     // a full k-tile of in-range values: fragments for step kk+1 are read from LDS while step kk is computed
-    auto plain_tile = [&]() {
+    auto plain_tile = [&]() __attribute__((always_inline)) {
         if constexpr (MODE != MODE_STD && TM == 4 && TN == 4) {
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;

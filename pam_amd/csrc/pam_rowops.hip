@@ -349,14 +349,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 // The chain of pad, sum, where, exp2, subtract, where, mul gradients in the order autograd
 // applies them (pam/cuda_bindings.py:78-97, 224-239, 43-57).
 struct Approx { bool a, b, e; };
+// all three gradients exact (the reference's default), as a type: the chain is then compiled without the choices
+struct ExactAll { static constexpr bool a = false, b = false, e = false; };
 
-__device__ __forceinline__ float softmax_dsum_term(float e, float total, float g, Offset o, Approx ap)
+template <class AP>
+__device__ __forceinline__ float softmax_dsum_term(float e, float total, float g, Offset o, AP ap)
 {
     if (ap.b) return -pam_mul_off(pad_div_off(pad_div_off(e, total, o.off, o.has), total, o.off, o.has), g, o.off, o.has);
     return pad_div_bwd(e, total, g, o.off, o.has);
 }
 
-__device__ __forceinline__ float softmax_dx(float xv, float e, float g, float inv, float dtotal, float shift, Offset o, Approx ap)
+template <class AP>
+__device__ __forceinline__ float softmax_dx(float xv, float e, float g, float inv, float dtotal, float shift, Offset o, AP ap)
 {
     const bool masked = f2u(xv) == 0xff800000u;
     float de = ap.a ? pam_mul_off(inv, g, o.off, o.has) : pam_mul_bwd(e, inv, g, 1.0f, false);
@@ -405,9 +409,9 @@ __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], c
 }
 
 // The same gradient with the checked primitives, for every combination of exact and approximate terms.
-template <int CH, class L>
-__device__ __forceinline__ void softmax_grad_row_checked(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
-                                                         float total, float inv, float shift, L& lay, long n, Offset o, Approx ap)
+template <int CH, class L, class AP>
+__device__ __forceinline__ void softmax_grad_row_checked_as(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
+                                                            float total, float inv, float shift, L& lay, long n, Offset o, AP ap)
 {
     float e[CH];
     float p = 0.0f;
@@ -420,9 +424,16 @@ __device__ __forceinline__ void softmax_grad_row_checked(const float (&xv)[CH], 
 #pragma unroll
     for (int c = 0; c < CH; ++c) out[c] = softmax_dx(xv[c], e[c], g[c], inv, dtotal, shift, o, ap);
 }
+template <int CH, class L>
+__device__ __forceinline__ void softmax_grad_row_checked(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
+                                                         float total, float inv, float shift, L& lay, long n, Offset o, Approx ap)
+{
+    if (!ap.a && !ap.b && !ap.e) softmax_grad_row_checked_as<CH>(xv, g, out, total, inv, shift, lay, n, o, ExactAll());
+    else softmax_grad_row_checked_as<CH>(xv, g, out, total, inv, shift, lay, n, o, ap);
+}
 
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC(CH)))) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC_GRAD(CH)))) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                               const float* __restrict__ row_sum, const float* __restrict__ shift_in,
                                                               float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
 {
