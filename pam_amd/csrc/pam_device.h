@@ -286,9 +286,11 @@ __device__ __forceinline__ float log2_entry_bwd(float x, float dy, float off, bo
 // returns -- or the chain has to be redone with the checked functions.
 struct Span {
     uint32_t lo = 0x7f7fffffu, hi = 0x00800000u;
+    uint32_t exp_arg = 0u;                        // largest magnitude given to pa_exp2_unchecked
     bool in_exp_range = true;
     __device__ __forceinline__ void see(uint32_t mag) { lo = min(lo, mag); hi = max(hi, mag); }
-    __device__ __forceinline__ bool normal() const { return in_exp_range && lo >= 0x00800000u && hi < kExpo; }
+    __device__ __forceinline__ bool normal() const
+    { return in_exp_range && lo >= 0x00800000u && hi < kExpo && exp_arg <= 0x42fc0000u; }     // |exp2 argument| <= 126
 };
 
 __device__ __forceinline__ float pam_unchecked(float a, float b, Span& sp)
@@ -317,16 +319,54 @@ __device__ __forceinline__ float pa_log2_unchecked(float x, Span& sp)
     sp.see(mag);
     return (float)((int)mag - (int)kBias) * 0x1p-23f;
 }
-// pa_exp2 for -126 <= floor(x) <= 127, where 2**floor(x) is a normal number
+// pa_exp2 for |x| <= 126, where 2**floor(x) is a normal number and so is the result (the arguments in
+// (126, 128), which would also do, are left to the checked function: one max per call instead of two compares)
 __device__ __forceinline__ float pa_exp2_unchecked(float x, Span& sp)
 {
-    sp.in_exp_range = sp.in_exp_range && (x >= -126.0f) && (x < 128.0f);       // false for NaN
+    sp.exp_arg = max(sp.exp_arg, f2u(x) & ~kSign);                             // NaN is larger than any bound
     float f = floorf(x);
     float t = (1.0f + x) - f;
     return u2f((uint32_t)((int)f + 127) << 23) * t;
 }
+// Without an offset t (*) 1 is t itself when t is a normal number: only that is recorded.
 __device__ __forceinline__ float exp2_entry_unchecked(float t, float off, bool has_off, Span& sp)
-{ return pa_exp2_unchecked(pam_unchecked_off(t, 1.0f, off, has_off, sp), sp); }
+{
+    if (!has_off) { sp.see(f2u(t) & ~kSign); return pa_exp2_unchecked(t, sp); }
+    return pa_exp2_unchecked(pam_unchecked_off(t, 1.0f, off, has_off, sp), sp);
+}
+
+// Cheaper forms for the usual places in a chain.  Each records its result and those operands that its name does not
+// excuse; for the excused ones the caller vouches: a constant, a value recorded earlier in the chain, a value that
+// is a normal number by construction (a result of pa_exp2_unchecked).
+// a (*) k, k a positive normal constant: records a and the result
+__device__ __forceinline__ float pam_unchecked_const(float a, float k, Span& sp)
+{
+    const uint32_t ai = f2u(a), ma = ai & ~kSign, s = ma + (f2u(k) - kBias);
+    sp.see(ma); sp.see(s);
+    return u2f(s | (ai & kSign));
+}
+// a (*) b, a recorded earlier: records b and the result
+__device__ __forceinline__ float pam_unchecked_seen(float a, float b, Span& sp)
+{
+    const uint32_t ai = f2u(a), bi = f2u(b), mb = bi & ~kSign, s = (ai & ~kSign) + mb - kBias;
+    sp.see(mb); sp.see(s);
+    return u2f(s | ((ai ^ bi) & kSign));
+}
+// a (*) a: records a and the result (which is positive)
+__device__ __forceinline__ float pam_unchecked_square(float a, Span& sp)
+{
+    const uint32_t ma = f2u(a) & ~kSign, s = ma + ma - kBias;
+    sp.see(ma); sp.see(s);
+    return u2f(s);
+}
+// a (/) b, b a positive normal number recorded by the caller, a recorded earlier (or normal by construction):
+// records the result
+__device__ __forceinline__ float pad_unchecked_by_positive(float a, float b, Span& sp)
+{
+    const uint32_t ai = f2u(a), s = (ai & ~kSign) - f2u(b) + kBias;            // a wrap lands above the exponent mask and is caught
+    sp.see(s);
+    return u2f(s | (ai & kSign));
+}
 __device__ __forceinline__ float log2_entry_unchecked(float v, float off, bool has_off, Span& sp)
 { return pad_unchecked_off(pa_log2_unchecked(v, sp), 1.0f, off, has_off, sp); }
 __device__ __forceinline__ float pow_half_unchecked(float v, float off, bool has_off, Span& sp)

@@ -217,6 +217,12 @@ struct Checked {
     // 0 (/) b for an element whose weight is exactly zero
     __device__ __forceinline__ float zero_over(float b) { return pad_div_off(0.0f, b, o.off, o.has); }
     __device__ __forceinline__ bool valid() const { return true; }
+    // the places where the unchecked arithmetic has cheaper forms
+    __device__ __forceinline__ float mul_const(float a, float k) { return mul(a, k); }
+    __device__ __forceinline__ float mul_seen(float a, float b) { return mul(a, b); }
+    __device__ __forceinline__ float square(float a) { return mul(a, a); }
+    __device__ __forceinline__ float div_by_positive(float a, float b) { return div(a, b); }
+    __device__ __forceinline__ void record(float) {}
 };
 struct Unchecked {
     Offset o; Span sp;
@@ -227,6 +233,14 @@ struct Unchecked {
     __device__ __forceinline__ float root(float v) { return pow_half_unchecked(v, o.off, o.has, sp); }
     __device__ __forceinline__ float zero_over(float) { return 0.0f; }      // the divisor is a positive normal number when valid
     __device__ __forceinline__ bool valid() const { return sp.normal(); }
+    // Cheaper forms (an offset takes the general ones).  mul_const: k is a positive normal constant; mul_seen and
+    // div_by_positive: a was recorded earlier in the chain or is a result of exp2; div_by_positive: b is not negative
+    // and was given to record().
+    __device__ __forceinline__ float mul_const(float a, float k) { return o.has ? mul(a, k) : pam_unchecked_const(a, k, sp); }
+    __device__ __forceinline__ float mul_seen(float a, float b) { return o.has ? mul(a, b) : pam_unchecked_seen(a, b, sp); }
+    __device__ __forceinline__ float square(float a) { return o.has ? mul(a, a) : pam_unchecked_square(a, sp); }
+    __device__ __forceinline__ float div_by_positive(float a, float b) { return o.has ? div(a, b) : pad_unchecked_by_positive(a, b, sp); }
+    __device__ __forceinline__ void record(float v) { sp.see(f2u(v) & ~kSign); }
 };
 __device__ __forceinline__ bool wave_valid(const Unchecked& u) { return __ballot(!u.valid()) == 0ull; }
 
@@ -245,16 +259,17 @@ __device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool masked = f2u(xv[c]) == 0xff800000u;       // computed on stand-in values, then replaced
-        const float t = m.mul(masked ? 1.0f : xv[c], kLog2E) - shift;
+        const float t = m.mul_const(masked ? 1.0f : xv[c], kLog2E) - shift;
         const float e = m.exp2(masked ? 0.5f : t);
         out[c] = masked ? 0.0f : e;
         p = p + out[c];
     }
-    const float total = lay.sum(p);
+    const float total = lay.sum(p);                  // a sum of weights from +0: never negative
+    m.record(total);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool masked = f2u(xv[c]) == 0xff800000u;
-        const float q = m.div(masked ? 1.0f : out[c], total);
+        const float q = m.div_by_positive(masked ? 1.0f : out[c], total);       // a weight is a result of exp2
         out[c] = masked ? m.zero_over(total) : q;
     }
     return total;
@@ -298,7 +313,7 @@ __device__ __forceinline__ void for_blocks2(const float* __restrict__ row_a, con
 template <class M>
 __device__ __forceinline__ float softmax_stream(const float* __restrict__ xr, float* __restrict__ yr, long n, int lane, float shift, M& m)
 {
-    auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
+    auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul_const(masked ? 1.0f : x, kLog2E) - shift); };
     float p = 0.0f;
     for_blocks(xr, (int)n, lane, kNegInf, [&](long, bool, float x) {
         const bool masked = f2u(x) == 0xff800000u;
@@ -306,9 +321,10 @@ __device__ __forceinline__ float softmax_stream(const float* __restrict__ xr, fl
         p = p + (masked ? 0.0f : e);
     });
     const float total = wave_sum(p);
+    m.record(total);
     for_blocks(xr, (int)n, lane, kNegInf, [&](long i, bool inside, float x) {
         const bool masked = f2u(x) == 0xff800000u;
-        const float q = m.div(masked ? 1.0f : weight(x, masked), total);
+        const float q = m.div_by_positive(masked ? 1.0f : weight(x, masked), total);
         if (inside) yr[i] = masked ? m.zero_over(total) : q;
     });
     return total;
@@ -502,7 +518,7 @@ __device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shif
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool inside = lay.index(c) < n;                    // lanes past the end work on stand-in values
-        const float t = m.mul(inside ? xv[c] : 1.0f, kLog2E) - shift;
+        const float t = m.mul_const(inside ? xv[c] : 1.0f, kLog2E) - shift;
         const float e = m.exp2(inside ? t : 0.5f);
         if (inside) p = p + e;
     }
@@ -536,7 +552,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             auto sweep = [&](auto& m) {
                 float p = 0.0f;
                 for_blocks(xr, (int)n, lane, 0.0f, [&](long, bool inside, float v) {
-                    const float e = m.exp2(inside ? m.mul(v, kLog2E) - shift : 0.5f);
+                    const float e = m.exp2(inside ? m.mul_const(v, kLog2E) - shift : 0.5f);
                     if (inside) p = p + e;
                 });
                 return m.div(shift + m.log2(wave_sum(p)), kLog2E);
@@ -576,15 +592,16 @@ __device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&ou
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         out[c] = xv[c] - mu;                                             // lanes past the end hold -mu, a stand-in
-        const float sq = m.mul(out[c], out[c]);
+        const float sq = m.square(out[c]);
         if (lay.index(c) < n) p = p + sq;
     }
-    const float denom = m.root(m.div(lay.sum(p), count) + eps);
+    const float denom = m.root(m.div(lay.sum(p), count) + eps);         // a result of exp2 (or the zero of the power): never negative
+    m.record(denom);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const long i = lay.index(c); const bool inside = i < n;
-        float r = m.div(out[c], denom);
-        if (weight) r = m.mul(r, inside ? weight[i] : 1.0f);
+        float r = m.div_by_positive(out[c], denom);                      // the centred value was recorded by square()
+        if (weight) r = m.mul_seen(r, inside ? weight[i] : 1.0f);
         if (bias) r = r + (inside ? bias[i] : 0.0f);
         out[c] = r;
     }
@@ -616,13 +633,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 const float mu = m.div(wave_sum(p), count);
                 p = 0.0f;
                 for_blocks(xr, (int)n, lane, 0.0f, [&](long, bool inside, float v) {
-                    const float c = v - mu, sq = m.mul(c, c);                                    // past the end: -mu, a stand-in
+                    const float c = v - mu, sq = m.square(c);                                    // past the end: -mu, a stand-in
                     if (inside) p = p + sq;
                 });
                 const float denom = m.root(m.div(wave_sum(p), count) + eps);
+                m.record(denom);
                 for_blocks(xr, (int)n, lane, 0.0f, [&](long i, bool inside, float v) {
-                    float r = m.div(v - mu, denom);
-                    if (weight) r = m.mul(r, inside ? weight[i] : 1.0f);
+                    float r = m.div_by_positive(v - mu, denom);                                  // v - mu was recorded by square()
+                    if (weight) r = m.mul_seen(r, inside ? weight[i] : 1.0f);
                     if (bias) r = r + (inside ? bias[i] : 0.0f);
                     if (inside) yr[i] = r;
                 });
