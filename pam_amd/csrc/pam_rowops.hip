@@ -180,6 +180,14 @@ __device__ __forceinline__ void load_row(float (&v)[CH], const float* __restrict
 #pragma unroll
     for (int c = 0; c < CH; ++c) { const long i = lay.index(c); v[c] = i < n ? p[i] : fill; }
 }
+// Register-resident rows, one wavefront per row, in logsumexp forward (one array of registers per row; the kernels
+// with two measured slower with it): the next row of the wavefront is fetched while the current one is computed.  Past the last row the fetch repeats the last row: a conditional fetch would tie the registers to their
+// old contents and make the compiler wait for them at once.
+#define PAM_WAVE_FIRST_ROW(AHEAD, X, FILL) load_row<CH>(AHEAD, X + (wave < rows ? wave : rows - 1) * n, n, lane, FILL)
+#define PAM_WAVE_NEXT_ROW(NOW, AHEAD, X, FILL)                                                           \
+    _Pragma("unroll") for (int c = 0; c < CH; ++c) NOW[c] = AHEAD[c];                                    \
+    load_row<CH>(AHEAD, X + (r + nwaves < rows ? r + nwaves : rows - 1) * n, n, lane, FILL)
+
 template <int CH, class L>
 __device__ __forceinline__ void store_row(const float (&v)[CH], float* __restrict__ p, long n, const L& lay)
 {
@@ -534,11 +542,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float shift = fold_shift<kWaves>(partial, partials);
     if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
+    float ahead[CH > 0 ? CH : 1];
+    if constexpr (CH > 0) PAM_WAVE_FIRST_ROW(ahead, x, 0.0f);
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
         if constexpr (CH > 0) {
             float xv[CH];
-            load_row<CH>(xv, xr, n, lane, 0.0f);
+            PAM_WAVE_NEXT_ROW(xv, ahead, x, 0.0f);
             WaveRow lay{lane};
             Unchecked u{o, Span()};
             float out = logsumexp_row<CH>(xv, shift, lay, n, u);
