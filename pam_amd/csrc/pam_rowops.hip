@@ -180,13 +180,17 @@ __device__ __forceinline__ void load_row(float (&v)[CH], const float* __restrict
 #pragma unroll
     for (int c = 0; c < CH; ++c) { const long i = lay.index(c); v[c] = i < n ? p[i] : fill; }
 }
-// Register-resident rows, one wavefront per row, in logsumexp forward (one array of registers per row; the kernels
-// with two measured slower with it): the next row of the wavefront is fetched while the current one is computed.  Past the last row the fetch repeats the last row: a conditional fetch would tie the registers to their
+// Register-resident rows, one wavefront per row, in the forward kernels (one array of registers per row; kernels
+// with two or three measured slower with it): the next row of the wavefront is fetched while the current one is computed.  Past the last row the fetch repeats the last row: a conditional fetch would tie the registers to their
 // old contents and make the compiler wait for them at once.
-#define PAM_WAVE_FIRST_ROW(AHEAD, X, FILL) load_row<CH>(AHEAD, X + (wave < rows ? wave : rows - 1) * n, n, lane, FILL)
-#define PAM_WAVE_NEXT_ROW(NOW, AHEAD, X, FILL)                                                           \
-    _Pragma("unroll") for (int c = 0; c < CH; ++c) NOW[c] = AHEAD[c];                                    \
-    load_row<CH>(AHEAD, X + (r + nwaves < rows ? r + nwaves : rows - 1) * n, n, lane, FILL)
+// ON (a compile-time choice per kernel and row length, by measurement) = false: the row is simply loaded.
+#define PAM_WAVE_FIRST_ROW(ON, AHEAD, X, FILL) \
+    if constexpr (ON) load_row<CH>(AHEAD, X + (wave < rows ? wave : rows - 1) * n, n, lane, FILL)
+#define PAM_WAVE_NEXT_ROW(ON, NOW, AHEAD, X, FILL)                                                       \
+    if constexpr (ON) {                                                                                  \
+        _Pragma("unroll") for (int c = 0; c < CH; ++c) NOW[c] = AHEAD[c];                                \
+        load_row<CH>(AHEAD, X + (r + nwaves < rows ? r + nwaves : rows - 1) * n, n, lane, FILL);         \
+    } else load_row<CH>(NOW, X + r * n, n, lane, FILL)
 
 template <int CH, class L>
 __device__ __forceinline__ void store_row(const float (&v)[CH], float* __restrict__ p, long n, const L& lay)
@@ -260,25 +264,28 @@ __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
 }
 
 // one row held in registers: weights, their sum, the quotients; masked (-inf) elements weigh exactly zero
+// The row is transformed in place (inputs, then weights, then quotients): one array of registers per row leaves
+// room to fetch the next row meanwhile.  A weight is never negative, so -1 marks the masked elements in between.
+constexpr uint32_t kMaskedMark = 0xbf800000u;
 template <int CH, class M, class L>
-__device__ __forceinline__ float softmax_row(const float (&xv)[CH], float (&out)[CH], float shift, M& m, L& lay)
+__device__ __forceinline__ float softmax_row(float (&v)[CH], float shift, M& m, L& lay)
 {
     float p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const bool masked = f2u(xv[c]) == 0xff800000u;       // computed on stand-in values, then replaced
-        const float t = m.mul_const(masked ? 1.0f : xv[c], kLog2E) - shift;
+        const bool masked = f2u(v[c]) == 0xff800000u;        // computed on stand-in values, then replaced
+        const float t = m.mul_const(masked ? 1.0f : v[c], kLog2E) - shift;
         const float e = m.exp2(masked ? 0.5f : t);
-        out[c] = masked ? 0.0f : e;
-        p = p + out[c];
+        v[c] = masked ? u2f(kMaskedMark) : e;
+        p = p + (masked ? 0.0f : e);
     }
     const float total = lay.sum(p);                  // a sum of weights from +0: never negative
     m.record(total);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const bool masked = f2u(xv[c]) == 0xff800000u;
-        const float q = m.div_by_positive(masked ? 1.0f : out[c], total);       // a weight is a result of exp2
-        out[c] = masked ? m.zero_over(total) : q;
+        const bool masked = f2u(v[c]) == kMaskedMark;
+        const float q = m.div_by_positive(masked ? 1.0f : v[c], total);         // a weight is a result of exp2
+        v[c] = masked ? m.zero_over(total) : q;
     }
     return total;
 }
@@ -348,18 +355,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float shift = fold_shift<kWaves>(partial, partials);
     if (wave == 0 && lane == 0) *shift_out = shift;
+    float ahead[CH > 0 ? CH : 1];
+    constexpr bool kAhead = CH >= 8;
+    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, kNegInf);                      // the fill has weight zero
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
         float total;
         if constexpr (CH > 0) {
-            float xv[CH], out[CH];
-            load_row<CH>(xv, xr, n, lane, kNegInf);            // the fill has weight zero
+            float v[CH];
+            PAM_WAVE_NEXT_ROW(kAhead, v, ahead, x, kNegInf);
             WaveRow lay{lane};
             Unchecked u{o, Span()};
-            total = softmax_row<CH>(xv, out, shift, u, lay);
-            if (!wave_valid(u)) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k, lay); }
-#pragma unroll
-            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
+            total = softmax_row<CH>(v, shift, u, lay);
+            if (!wave_valid(u)) {                              // the row is read again (from cache)
+                load_row<CH>(v, xr, n, lane, kNegInf);
+                Checked k{o}; total = softmax_row<CH>(v, shift, k, lay);
+            }
+            store_row<CH>(v, yr, n, lay);
         } else {
             Unchecked u{o, Span()};
             total = softmax_stream(xr, yr, n, lane, shift, u);
@@ -543,12 +555,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     const float shift = fold_shift<kWaves>(partial, partials);
     if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
     float ahead[CH > 0 ? CH : 1];
-    if constexpr (CH > 0) PAM_WAVE_FIRST_ROW(ahead, x, 0.0f);
+    constexpr bool kAhead = CH > 0;
+    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, 0.0f);
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
         if constexpr (CH > 0) {
             float xv[CH];
-            PAM_WAVE_NEXT_ROW(xv, ahead, x, 0.0f);
+            PAM_WAVE_NEXT_ROW(kAhead, xv, ahead, x, 0.0f);
             WaveRow lay{lane};
             Unchecked u{o, Span()};
             float out = logsumexp_row<CH>(xv, shift, lay, n, u);
@@ -591,18 +604,19 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restr
 
 // ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
 template <int CH, class M, class L>
-__device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&out)[CH], const float* __restrict__ weight,
-                                               const float* __restrict__ bias, L& lay, long n, float count, float eps, M& m)
+__device__ __forceinline__ void layer_norm_row(float (&v)[CH], const float* __restrict__ weight, const float* __restrict__ bias,
+                                               L& lay, long n, float count, float eps, M& m)
 {
+    // in place: inputs, then centred values, then results (one array of registers per row)
     float p = 0.0f;
 #pragma unroll
-    for (int c = 0; c < CH; ++c) p = p + xv[c];                          // the fill adds +0
+    for (int c = 0; c < CH; ++c) p = p + v[c];                           // the fill adds +0
     const float mu = m.div(lay.sum(p), count);
     p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        out[c] = xv[c] - mu;                                             // lanes past the end hold -mu, a stand-in
-        const float sq = m.square(out[c]);
+        v[c] = v[c] - mu;                                                // lanes past the end hold -mu, a stand-in
+        const float sq = m.square(v[c]);
         if (lay.index(c) < n) p = p + sq;
     }
     const float denom = m.root(m.div(lay.sum(p), count) + eps);         // a result of exp2 (or the zero of the power): never negative
@@ -610,10 +624,10 @@ __device__ __forceinline__ void layer_norm_row(const float (&xv)[CH], float (&ou
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const long i = lay.index(c); const bool inside = i < n;
-        float r = m.div_by_positive(out[c], denom);                      // the centred value was recorded by square()
+        float r = m.div_by_positive(v[c], denom);                        // the centred value was recorded by square()
         if (weight) r = m.mul_seen(r, inside ? weight[i] : 1.0f);
         if (bias) r = r + (inside ? bias[i] : 0.0f);
-        out[c] = r;
+        v[c] = r;
     }
 }
 
@@ -625,17 +639,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float count = (float)n;
+    float ahead[CH > 0 ? CH : 1];
+    constexpr bool kAhead = false;                         // measured slower with it
+    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, 0.0f);
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
         if constexpr (CH > 0) {
-            float xv[CH], out[CH];
-            load_row<CH>(xv, xr, n, lane, 0.0f);
+            float v[CH];
+            PAM_WAVE_NEXT_ROW(kAhead, v, ahead, x, 0.0f);
             WaveRow lay{lane};
             Unchecked u{o, Span()};
-            layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, u);
-            if (!wave_valid(u)) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, k); }
-#pragma unroll
-            for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) yr[i] = out[c]; }
+            layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, u);
+            if (!wave_valid(u)) {                              // the row is read again (from cache)
+                load_row<CH>(v, xr, n, lane, 0.0f);
+                Checked k{o}; layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, k);
+            }
+            store_row<CH>(v, yr, n, lay);
         } else {
             auto sweep = [&](auto& m) {
                 float p = 0.0f;
@@ -1009,15 +1028,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >
 #else
 #define PAM_BLOCK_ATTR
 #endif
-// logsumexp forward, which needs the fewest registers: the input row of the next iteration is fetched while the
-// current one is computed (there is one work-group per compute unit, so nothing else would hide the latency;
-// the other kernels have no registers to spare for it).  Past the last row the fetch repeats the last row:
+// The forward kernels, which hold one array of registers per row: the input row of the next iteration is fetched
+// while the current one is computed (there is one work-group per compute unit, so nothing else would hide the
+// latency; the gradient kernels have no registers to spare for it).  Past the last row the fetch repeats the last row:
 // a conditional fetch would tie the registers to their old contents and make the compiler wait for them at once.
-#define PAM_BLOCK_FIRST_ROW(AHEAD, X, FILL) \
-    load_row<CH>(AHEAD, X + (blockIdx.x < rows ? (long)blockIdx.x : rows - 1) * n, n, lay, FILL)
-#define PAM_BLOCK_NEXT_ROW(NOW, AHEAD, X, FILL)                                                          \
-    _Pragma("unroll") for (int c = 0; c < CH; ++c) NOW[c] = AHEAD[c];                                    \
-    load_row<CH>(AHEAD, X + (r + gridDim.x < rows ? r + gridDim.x : rows - 1) * n, n, lay, FILL)
+#define PAM_BLOCK_FIRST_ROW(ON, AHEAD, X, FILL) \
+    if constexpr (ON) load_row<CH>(AHEAD, X + (blockIdx.x < rows ? (long)blockIdx.x : rows - 1) * n, n, lay, FILL)
+#define PAM_BLOCK_NEXT_ROW(ON, NOW, AHEAD, X, FILL)                                                      \
+    if constexpr (ON) {                                                                                  \
+        _Pragma("unroll") for (int c = 0; c < CH; ++c) NOW[c] = AHEAD[c];                                \
+        load_row<CH>(AHEAD, X + (r + gridDim.x < rows ? r + gridDim.x : rows - 1) * n, n, lay, FILL);    \
+    } else load_row<CH>(NOW, X + r * n, n, lay, FILL)
 #define PAM_BLOCK_ROW_SETUP                                                        \
     __shared__ float red_slots[2][kBlockWaves];                                    \
     BlockRow lay{(int)threadIdx.x, red_slots, 0};                                  \
@@ -1033,13 +1054,19 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_fwd_bloc
     PAM_BLOCK_ROW_SETUP;
     const float shift = fold_shift<kBlockWaves>(partial, partials);
     if (blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
+    float ahead[CH];
+    constexpr bool kAhead = CH >= 16;
+    PAM_BLOCK_FIRST_ROW(kAhead, ahead, x, kNegInf);
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
-        float xv[CH], out[CH];
-        load_row<CH>(xv, x + r * n, n, lay, kNegInf);
+        float v[CH];
+        PAM_BLOCK_NEXT_ROW(kAhead, v, ahead, x, kNegInf);
         Unchecked u{o, Span()};
-        float total = softmax_row<CH>(xv, out, shift, u, lay);
-        if (!lay.all(u.valid())) { Checked k{o}; total = softmax_row<CH>(xv, out, shift, k, lay); }
-        store_row<CH>(out, y + r * n, n, lay);
+        float total = softmax_row<CH>(v, shift, u, lay);
+        if (!lay.all(u.valid())) {                             // the row is read again (from cache)
+            load_row<CH>(v, x + r * n, n, lay, kNegInf);
+            Checked k{o}; total = softmax_row<CH>(v, shift, k, lay);
+        }
+        store_row<CH>(v, y + r * n, n, lay);
         if (threadIdx.x == 0) row_sum[r] = total;
     }
 }
@@ -1076,10 +1103,10 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_block_
     const float shift = fold_shift<kBlockWaves>(partial, partials);
     if (shift_out && blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     float ahead[CH];
-    PAM_BLOCK_FIRST_ROW(ahead, x, 0.0f);
+    PAM_BLOCK_FIRST_ROW(true, ahead, x, 0.0f);
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float xv[CH];
-        PAM_BLOCK_NEXT_ROW(xv, ahead, x, 0.0f);
+        PAM_BLOCK_NEXT_ROW(true, xv, ahead, x, 0.0f);
         Unchecked u{o, Span()};
         float out = logsumexp_row<CH>(xv, shift, lay, n, u);
         if (!lay.all(u.valid())) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lay, n, k); }
@@ -1113,13 +1140,19 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_fwd_b
 {
     PAM_BLOCK_ROW_SETUP;
     const float count = (float)n;
+    float ahead[CH];
+    constexpr bool kAhead = false;                         // measured slower with it
+    PAM_BLOCK_FIRST_ROW(kAhead, ahead, x, 0.0f);
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
-        float xv[CH], out[CH];
-        load_row<CH>(xv, x + r * n, n, lay, 0.0f);
+        float v[CH];
+        PAM_BLOCK_NEXT_ROW(kAhead, v, ahead, x, 0.0f);
         Unchecked u{o, Span()};
-        layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, u);
-        if (!lay.all(u.valid())) { Checked k{o}; layer_norm_row<CH>(xv, out, weight, bias, lay, n, count, eps, k); }
-        store_row<CH>(out, y + r * n, n, lay);
+        layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, u);
+        if (!lay.all(u.valid())) {                             // the row is read again (from cache)
+            load_row<CH>(v, x + r * n, n, lay, 0.0f);
+            Checked k{o}; layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, k);
+        }
+        store_row<CH>(v, y + r * n, n, lay);
     }
 }
 
