@@ -961,9 +961,6 @@ void launch_kinds(int lk, int rk, dim3 grid, hipStream_t st, const GemmArgs& g, 
 #define PAM_GEMM_CASE(LK, RK) \
     if (lk == LK && rk == RK) { hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 4, BK, MODE, LK, RK>), grid, dim3(256), 0, st, g, partial); return; }
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC)
-#ifdef PAM_GEMM_FEW
-    return;
-#endif
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
@@ -1037,13 +1034,9 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
     float* partial = (float*)workspace;
     switch (mode) {
     case MODE_PAM: launch_mode<MODE_PAM>(p, lk, rk, st, g, batch, partial); break;
-#ifndef PAM_GEMM_FEW
     case MODE_STD: launch_mode<MODE_STD>(p, lk, rk, st, g, batch, partial); break;
     case MODE_BWD_DL: launch_mode<MODE_BWD_DL>(p, lk, rk, st, g, batch, partial); break;
     default: launch_mode<MODE_BWD_DR>(p, lk, rk, st, g, batch, partial); break;
-#else
-    default: return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "%s: experimental build without this mode", what);
-#endif
     }
     if (p.ksplit > 1) {
         long slab = batch * M * N;

@@ -985,9 +985,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     }
 }
 
-// dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias
+// dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias.  Rows of 1024 values: three
+// wavefronts per SIMD (168 registers); left at two the compiler takes 181 and a third fewer wavefronts fit.
 template <int CH>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >= 16 ? 2 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >= 16 ? 3 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
     float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
 {
