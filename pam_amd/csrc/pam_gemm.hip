@@ -24,15 +24,17 @@
 //    long k and 16 deep for short k.
 //  * The bias subtraction and the optional offset (R' = R (*) offset) are applied once per
 //    element while staging R.
-//  * While staging, every element's exponent is folded into a running min/max.  If all of a
-//    k-tile's L and R values are normal numbers with magnitude in [2^-63, 2^64), no product
-//    in the tile can leave the normal range and the two-instruction loop is exact;
-//    a k-tile that only adds zeros to that in one operand (ReLU activations, padding) keeps two
-//    instructions per product: the zero becomes a stand-in value and the accumulating fma
-//    multiplies the product by 0 or 1; zeros in both operands cost one select per product;
-//    anything else (subnormals, inf, NaN, extreme exponents) takes a guarded loop that
-//    evaluates the full definition per product on operands decomposed once per k-step.
-//    The choice is uniform per work-group and k-tile.
+//  * Staging begins with a quick test, one shift-add per value folded by max: if all of a k-tile's L and R
+//    values are normal numbers with magnitude in [2^-63, 2^64), no product in the tile can leave the normal
+//    range and the two-instruction loop is exact; such a tile is stored as it is.  Only a tile that fails is
+//    classified value by value.  Its full k-tiles that only add zeros to that (ReLU activations, padding,
+//    pruned weights) keep two instructions per product and skip the products with a zero under the
+//    execution mask (a PAM product with a zero is +0, and adding it changes nothing); anything else
+//    (subnormals, inf, NaN, extreme exponents) takes a guarded loop that evaluates the full definition
+//    per product on operands decomposed once per k-step.  The choice is uniform per work-group and k-tile.
+//  * The products of a full in-range k-tile are written out in assembly, sixteen per k-step, and take the
+//    LDS addresses as in-out operands: given the unrolled k-tile as one block, the compiler issues all of
+//    its LDS reads first and spills.
 //  * Rows beyond M / N are clamped to the last valid row when loading (their results are
 //    never stored); the k tail runs a shorter loop, padding never enters the arithmetic.
 //  * Shapes with few output tiles and long k (dX: 12608 x 192, k = 768; dW: 192 x 768,

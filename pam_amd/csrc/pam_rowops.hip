@@ -6,11 +6,14 @@
 // (pam/cuda_bindings.py:27-57, 66-97, 210-239); what is fused away is the traffic: the
 // unfused chain moves every intermediate through HBM (68 B per element for softmax),
 // here a row is read once from HBM (again from cache for the second sweep) and written
-// once.  One wavefront owns a row: lane l takes the elements l, l + 64, l + 128, ...
+// once.  One wavefront owns a row: lane l takes the elements l, l + 64, l + 128, ...;
+// rows of 4097 ... 16384 values are owned by a work-group of 1024 threads instead
+// (thread t takes t, t + 1024, ...), which holds the row in registers too.
 //
 // The reference leaves the order of its row sums to torch.sum.  Here the order is fixed:
 // lane l adds its elements in ascending order starting from +0, then the 64 partial sums
-// are combined by a butterfly, p[l] = p[l] + p[l ^ s] for s = 32, 16, 8, 4, 2, 1.
+// are combined by a butterfly, p[l] = p[l] + p[l ^ s] for s = 32, 16, 8, 4, 2, 1; a
+// work-group's 16 wavefront sums are then added in ascending order.
 // All kernels are HBM-bound streams: 12 B/element for softmax forward (4 for the global
 // maximum sweep, 4 in, 4 out), 12 for its backward, 8 for layer_norm and log_softmax.
 #include <math.h>
