@@ -34,10 +34,18 @@ def parse():
     return ap.parse_args()
 
 
-def event_time_ms(fn, iters, torch):
-    """Average duration of fn() over `iters` back-to-back launches, HIP events on the launch stream."""
+def event_time_ms(fn, iters, torch, settle_s=0.03):
+    """Average duration of fn() over `iters` back-to-back launches, HIP events on the launch stream.  The same launches
+    run for `settle_s` first: the operands of a row are made on the host while the GPU idles, and the first
+    milliseconds after an idle period run at lower clocks (a 130 us product measured 146 us with seven warm-up launches
+    and 122 us after 30 ms of them)."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     fn(); torch.cuda.synchronize()
+    t_end = time.perf_counter() + settle_s
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(max(3, iters // 4)):        # untimed launches ahead of the start event: the queue is full when timing begins
         fn()
     start.record()
