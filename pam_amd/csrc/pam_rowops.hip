@@ -1049,8 +1049,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >
     const int lane = threadIdx.x % 64;                                             \
     (void)lane
 
+// Up to 12 values per thread the kernel fits 64 registers: two work-groups per compute unit.
 template <int CH>
-__global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_fwd_block_kernel(const float* __restrict__ x, float* __restrict__ y,
+__global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(CH <= 12 ? 8 : 4))) void softmax_fwd_block_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                                          float* __restrict__ row_sum, float* __restrict__ shift_out,
                                                                          long rows, long n, Offset o,
                                                                          const float* __restrict__ partial, int partials)
@@ -1107,10 +1108,11 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_block_
     const float shift = fold_shift<kBlockWaves>(partial, partials);
     if (shift_out && blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     float ahead[CH];
-    PAM_BLOCK_FIRST_ROW(true, ahead, x, 0.0f);
+    constexpr bool kAhead = CH < 16;                       // sixteen values per thread twice over would spill
+    PAM_BLOCK_FIRST_ROW(kAhead, ahead, x, 0.0f);
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float xv[CH];
-        PAM_BLOCK_NEXT_ROW(true, xv, ahead, x, 0.0f);
+        PAM_BLOCK_NEXT_ROW(kAhead, xv, ahead, x, 0.0f);
         Unchecked u{o, Span()};
         float out = logsumexp_row<CH>(xv, shift, lay, n, u);
         if (!lay.all(u.valid())) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lay, n, k); }
