@@ -341,6 +341,37 @@ def test_gpu_long_rows_with_special_values(oracle, off):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows,n", [(20000, 520), (1100, 4100)])
+def test_gpu_more_rows_than_the_launch_holds(oracle, rows, n):
+    """More rows than wavefronts (work-groups) in the launch: every wavefront (work-group) walks several rows, the
+    forward kernels fetching the next row while they compute the current one."""
+    x = rows_case(rows + n, rows, n)
+    g = np.random.RandomState(4).standard_normal(x.shape).astype(np.float32)
+    xt = _dev(x).requires_grad_()
+    y = pam_amd.softmax(xt, dim=-1, approx_bwd=True)
+    want, row_sum, shift = oracle.softmax_fwd(x)
+    assert_same_bits(y.detach().cpu().numpy(), want, "softmax")
+    y.backward(_dev(g))
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, None, (True, True, True)), "softmax gradient")
+    xf = rows_case(rows + n + 1, rows, n, masks=False)
+    lse, ls = oracle.logsumexp_fwd(xf, None, with_log_softmax=True)
+    xt = _dev(xf).requires_grad_()
+    y = pam_amd.log_softmax(xt, dim=-1, approx_bwd=True)
+    assert_same_bits(y.detach().cpu().numpy(), ls, "log_softmax")
+    y.backward(_dev(g))
+    sh = np.floor(oracle.pam(xf, C).max())
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g, sh, None, (True, True, True), log_softmax=True), "log_softmax gradient")
+    assert_same_bits(pam_amd.logsumexp(_dev(xf), dim=-1).cpu().numpy(), lse, "logsumexp")
+    w = (np.random.RandomState(6).standard_normal(n) + 2).astype(np.float32); b = np.random.RandomState(7).standard_normal(n).astype(np.float32)
+    xt = _dev(xf).requires_grad_()
+    y = pam_amd.layer_norm(xt, n, _dev(w), _dev(b), approx_bwd=True)
+    assert_same_bits(y.detach().cpu().numpy(), oracle.layer_norm_fwd(xf, w, b, 1e-5), "layer_norm")
+    y.backward(_dev(g))
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.layer_norm_bwd(xf, w, g, 1e-5, None, (True, True, True))[0], "layer_norm gradient")
+    assert_same_bits(pam_amd.mean(_dev(xf), dim=-1).cpu().numpy(), oracle.row_mean_fwd(xf), "mean")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_logsumexp_mean_layer_norm(oracle, off):
     for rows, n in [(1, 1), (3, 7), (4, 64), (50, 192), (2, 513), (33, 512), (2, 4096), (3, 4097), (3, 8193), (3, 10000), (2, 12289), (2, 16384), (2, 16385)]:
