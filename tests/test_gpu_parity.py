@@ -366,6 +366,16 @@ def test_deit_linear_full_size(K, oracle):
     dW2 = K.pam_matmul_fwd(dev(X2).T, dev(dY2), False, True, 1.0)
     cols2 = rng.choice(192, 16, replace=False)
     assert_same_bits(host(dW2)[:, cols2], ogemm(oracle, X2.T, dY2[:, cols2], plan_shape=(1, 768, 192, 12608)), "dW cols, 768 -> 192")
+    # the same layer behind a ReLU (half of the left operand's values are zeros: k-tiles that skip the zero products),
+    # then with 30 % of the weights pruned too (zeros in both operands)
+    X2r = np.maximum(X2, 0.0).astype(np.float32)
+    Y2r = K.pam_matmul_fwd(dev(X2r), dev(W2).T, True, False, 1.0)
+    assert_same_bits(host(Y2r)[rows], ogemm(oracle, X2r[rows], W2.T, plan_shape=(1, 12608, 192, 768)), "Y rows, ReLU input")
+    dW2r = K.pam_matmul_fwd(dev(X2r).T, dev(dY2), False, True, 1.0)
+    assert_same_bits(host(dW2r)[:, cols2], ogemm(oracle, X2r.T, dY2[:, cols2], plan_shape=(1, 768, 192, 12608)), "dW cols, ReLU input")
+    W2s = (W2 * (rng.rand(*W2.shape) >= 0.3)).astype(np.float32)
+    Y2s = K.pam_matmul_fwd(dev(X2r), dev(W2s).T, True, False, 1.0)
+    assert_same_bits(host(Y2s)[rows], ogemm(oracle, X2r[rows], W2s.T, plan_shape=(1, 12608, 192, 768)), "Y rows, ReLU input, pruned weight")
     # multiplying an operand by a power of two multiplies every PAM product, hence the sum, exactly
     assert torch.equal(K.pam_matmul_fwd(tX * 4.0, tW.T, True, False, 1.0), Y * 4.0)
     assert torch.equal(K.pam_matmul_fwd(tX, (tW * 0.5).T, True, False, 1.0), Y * 0.5)
