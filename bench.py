@@ -239,6 +239,9 @@ def main():
         # zeros in both operands: the same input against a weight matrix with 30 % of its entries pruned
         W2s = W2 * (torch.rand(W2.shape, generator=g) >= 0.3).to(dev)
         exact["fwd_12608x192x768_relu_input_pruned_weight"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2r, W2s.T, True, False, 1.0))
+        # one value in a thousand of the left operand a subnormal number: its k-step takes the full definition, the rest of its k-tile not
+        X2n = torch.where((torch.rand(X2.shape, generator=g) < 1e-3).to(dev), torch.full_like(X2, 1e-40), X2)
+        exact["fwd_12608x192x768_0.1pct_subnormal_input"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2n, W2.T, True, False, 1.0))
         for name, (ops, macs, fn) in exact.items():
             ms = event_time_ms(fn, 30, torch)
             other[name] = {"ms": round(ms, 4), "gmacs": round(macs / ms / 1e6, 1), "valu_frac": round(ops * macs / (ms * 1e-3) / lane_peak, 4)}

@@ -265,6 +265,42 @@ def test_matmul_exact_backward(K, oracle, delta_l, zeros, specials):
                 assert_same_bits(got, want, f"{ll} x {lr} off={off}")
 
 
+def _sparse_specials(shape, seed, every=600, zero_band=None):
+    """N(0,1) with one value in `every` outside the plain range (subnormal, inf, NaN, huge, tiny) at seeded places, and
+    zeros in a band of the k dimension: k-tiles then hold k-steps of every kind next to each other."""
+    rng = np.random.RandomState(seed)
+    x = rng.standard_normal(shape).astype(np.float32)
+    flat = x.reshape(-1)
+    idx = rng.choice(flat.size, size=max(3, flat.size // every), replace=False)
+    flat[idx] = np.resize(np.array([1e-40, 2.0 ** 100, -1e-39, np.inf, 2.0 ** -100, 3e38, np.nan], np.float32), idx.size)
+    if zero_band is not None:
+        axis, lo, hi = zero_band
+        band = [slice(None)] * x.ndim; band[axis] = slice(lo, hi)
+        sub = x[tuple(band)]
+        sub[rng.rand(*sub.shape) < 0.3] = 0.0
+    return x
+
+
+def test_matmul_few_specials_per_k_tile(K, oracle):
+    """A value that needs the full definition sends only its own k-step of the k-tile there; the other steps of the tile
+    take the plain form, or the zero-replacing one where the tile also holds zeros.  All layouts, forward and both exact
+    gradients, k = 256 (32-deep tiles) and 100 (16-deep, ragged)."""
+    for k in (256, 100):
+        A = _sparse_specials((150, k), 40 + k, zero_band=(1, 40, 90))
+        B = _sparse_specials((k, 90), 41 + k, zero_band=(0, 70, 100))
+        want = ogemm(oracle, A, B)
+        for la, ta in _layouts(A).items():
+            for lb, tb in _layouts(B).items():
+                assert_same_bits(host(K.pam_matmul_fwd(ta, tb, True, True, 1.0)), want, f"k={k} {la} x {lb}")
+        assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), ogemm(oracle, A, B, offset=1.0552), "offset")
+        D = _sparse_specials((150, 90), 42 + k, every=900)
+        for delta_l, mode in ((True, oracle.MODE_BWD_DELTA_L), (False, oracle.MODE_BWD_DELTA_R)):
+            want = ogemm(oracle, A, B, mode=mode, D=D)
+            for la, ta in _layouts(A).items():
+                for lb, tb in _layouts(B).items():
+                    assert_same_bits(host(K.pam_matmul_bwd(ta, tb, dev(D), True, True, delta_l, 1.0)), want, f"exact k={k} {la} x {lb}")
+
+
 def test_bmm_tails_and_strides(K, oracle):
     # the reference's own bmm test shape (pam/test_pam.py:198-205): power-of-two weights => equals bmm
     rng = np.random.RandomState(6)
