@@ -28,20 +28,25 @@ def parse():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-ms", type=float, default=30.0,
+                    help="each timed row first runs its launches for this long (0 for counter-collecting profiler passes)")
     ap.add_argument("--no-elementwise", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 2^26 floats (calibrates FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
-def event_time_ms(fn, iters, torch, settle_s=0.03):
+SETTLE_S = 0.03
+
+
+def event_time_ms(fn, iters, torch, settle_s=None):
     """Average duration of fn() over `iters` back-to-back launches, HIP events on the launch stream.  The same launches
     run for `settle_s` first: the operands of a row are made on the host while the GPU idles, and the first
     milliseconds after an idle period run at lower clocks (a 130 us product measured 146 us with seven warm-up launches
     and 122 us after 30 ms of them)."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     fn(); torch.cuda.synchronize()
-    t_end = time.perf_counter() + settle_s
+    t_end = time.perf_counter() + (SETTLE_S if settle_s is None else settle_s)
     while time.perf_counter() < t_end:
         for _ in range(8):
             fn()
@@ -80,7 +85,9 @@ def config1_operand(n, seed, torch, dev):
 
 
 def main():
+    global SETTLE_S
     args = parse()
+    SETTLE_S = args.settle_ms / 1e3
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
                  "(the path has no collective: it shards by rows, with one all-reduce of dW per layer)")
