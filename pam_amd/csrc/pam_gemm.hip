@@ -32,7 +32,7 @@
 //    execution mask (a PAM product with a zero is +0, and adding it changes nothing); anything else
 //    (subnormals, inf, NaN, extreme exponents) makes its k-tile choose per k-step: the steps that hold such
 //    a value evaluate the full definition per product on operands decomposed once per k-step, the others
-//    take the plain or the zero-replacing form.  The choices are uniform per work-group.
+//    take the plain form, or the zero-replacing one if the tile holds zeros too.  The choices are uniform per work-group.
 //  * The products of a full in-range k-tile are written out in assembly, sixteen per k-step, and take the
 //    LDS addresses as in-out operands: given the unrolled k-tile as one block, the compiler issues all of
 //    its LDS reads first and spills.
@@ -109,19 +109,6 @@ struct Stager {
     static constexpr bool kTakesOffset = (MODE == MODE_PAM && IS_R) || kSlopeSide;
     uint32_t emin = 255u, emax = 0u;
     bool bad = false, zero = false;
-    uint32_t odd_k = 0u, zero_k = 0u;             // per k of the tile: a value that needs the full definition / a zero
-
-    // the same, also recording under which k of the tile the value sits
-    __device__ __forceinline__ uint32_t one(float v, int k)
-    {
-        const uint32_t u = f2u(v), e = (u >> 23) & 0xffu;
-        const bool z = (u & ~kSign) == 0;
-        if (MODE != MODE_STD) {
-            odd_k |= (uint32_t)(!z && e - 64u > 126u) << k;
-            if (MODE == MODE_PAM) zero_k |= (uint32_t)z << k;
-        }
-        return one(v);
-    }
     __device__ __forceinline__ uint32_t one(float v)
     {
         uint32_t u = f2u(v);
@@ -154,7 +141,6 @@ template <bool ADDS>
 struct PlainStager {
     uint32_t add;
     __device__ __forceinline__ uint32_t one(float v) const { return ADDS ? f2u(v) + add : f2u(v); }
-    __device__ __forceinline__ uint32_t one(float v, int) const { return one(v); }
 };
 
 // Quick test of a staged value: (bits << 1) - (64 << 24) is below 127 << 24 exactly for the normal numbers
@@ -272,6 +258,33 @@ struct TileLoader {
         }
     }
 
+    // For a k-tile that holds a value in need of the full definition (rare): under which k of the tile the lane's
+    // values of that kind sit, bit k for k.  The same walk over the register tile as store().
+    __device__ __forceinline__ void odd_by_k(int tid, uint32_t& odd) const
+    {
+        auto see = [&](float f, int k) __attribute__((always_inline)) {
+            const uint32_t u = f2u(f), e = (u >> 23) & 0xffu;
+            odd |= (uint32_t)((u & ~kSign) != 0 && e - 64u > 126u) << k;
+        };
+        if (KIND == LOAD_KVEC) {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                const int k = ((tid + i * NT) % (BK / 4)) * 4;
+                see(v[i].x, k); see(v[i].y, k + 1); see(v[i].z, k + 2); see(v[i].w, k + 3);
+            }
+        } else if (KIND == LOAD_RVEC) {
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                const int k = (tid + i * NT) / (ROWS / 4);
+                see(v[i].x, k); see(v[i].y, k); see(v[i].z, k); see(v[i].w, k);
+            }
+        } else {
+            const float* s = reinterpret_cast<const float*>(v);
+#pragma unroll
+            for (int i = 0; i < kElems; ++i) see(s[i], (tid + i * NT) / ROWS);
+        }
+    }
+
     template <class S>
     __device__ __forceinline__ void store(uint32_t* lds, int tid, S& st)
     {
@@ -280,26 +293,24 @@ struct TileLoader {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
-                const int k = (id % (BK / 4)) * 4;
-                uint32_t* d = lds + k * LD + id / (BK / 4);
-                d[0 * LD] = st.one(v[i].x, k); d[1 * LD] = st.one(v[i].y, k + 1);
-                d[2 * LD] = st.one(v[i].z, k + 2); d[3 * LD] = st.one(v[i].w, k + 3);
+                uint32_t* d = lds + ((id % (BK / 4)) * 4) * LD + id / (BK / 4);
+                d[0 * LD] = st.one(v[i].x); d[1 * LD] = st.one(v[i].y);
+                d[2 * LD] = st.one(v[i].z); d[3 * LD] = st.one(v[i].w);
             }
         } else if (KIND == LOAD_RVEC) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
-                const int k = id / (ROWS / 4);
                 uint4 w;
-                w.x = st.one(v[i].x, k); w.y = st.one(v[i].y, k); w.z = st.one(v[i].z, k); w.w = st.one(v[i].w, k);
-                *reinterpret_cast<uint4*>(lds + k * LD + (id % (ROWS / 4)) * 4) = w;
+                w.x = st.one(v[i].x); w.y = st.one(v[i].y); w.z = st.one(v[i].z); w.w = st.one(v[i].w);
+                *reinterpret_cast<uint4*>(lds + (id / (ROWS / 4)) * LD + (id % (ROWS / 4)) * 4) = w;
             }
         } else {                                    // LOAD_ANY and LOAD_CONV: lane-consecutive rows
             const float* s = reinterpret_cast<const float*>(v);
 #pragma unroll
             for (int i = 0; i < kElems; ++i) {
                 int id = tid + i * NT;
-                lds[(id / ROWS) * LD + id % ROWS] = st.one(s[i], id / ROWS);
+                lds[(id / ROWS) * LD + id % ROWS] = st.one(s[i]);
             }
         }
     }
@@ -504,7 +515,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     __shared__ __attribute__((aligned(16))) uint32_t lds_l[2][BK * LDL];
     __shared__ __attribute__((aligned(16))) uint32_t lds_r[2][BK * LDR];
     __shared__ uint32_t lds_flag[2][NW];
-    __shared__ uint32_t lds_odd_k[2][NW], lds_zero_k[2][NW];       // per k of a tile that is not plain: see Stager
+    __shared__ uint32_t lds_odd_k[2][NW];         // bit k: some value under k of the tile needs the full definition
 
     const int tid = threadIdx.x, tx = tid % TXN, ty = tid / TXN;
     const int wave = tid / 64, lane = tid % 64;
@@ -577,11 +588,17 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         rl.store(lds_r[buf], tid, sr);
         const uint32_t found = (__ballot(sl.out_of_range() || sr.out_of_range()) != 0ull ? kGuarded : 0u)
                              | (__ballot(sl.zero) != 0ull ? kZerosL : 0u) | (__ballot(sr.zero) != 0ull ? kZerosR : 0u);
-        // which k of the tile hold such values: the loop for this tile chooses per k-step
-        uint32_t odd = sl.odd_k | sr.odd_k, zer = sl.zero_k | sr.zero_k;
+        if (lane == 0) lds_flag[buf][wave] = found;
+        // A wavefront that found such a value (rare) walks its register tile once more and records under which k
+        // they sit: the loop for this tile chooses per k-step.  The other wavefronts have none to report.
+        uint32_t odd = 0u;
+        if (__builtin_expect(found >= kGuarded, 0)) {
+            ll.odd_by_k(tid, odd);
+            rl.odd_by_k(tid, odd);
 #pragma unroll
-        for (int s = 32; s >= 1; s >>= 1) { odd |= __shfl_xor(odd, s, 64); zer |= __shfl_xor(zer, s, 64); }
-        if (lane == 0) { lds_flag[buf][wave] = found; lds_odd_k[buf][wave] = odd; lds_zero_k[buf][wave] = zer; }
+            for (int s = 32; s >= 1; s >>= 1) odd |= __shfl_xor(odd, s, 64);
+        }
+        if (lane == 0) lds_odd_k[buf][wave] = odd;
     };
 
     if (ktiles > 0) {
@@ -823,14 +840,15 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             for (int kk = 0; kk < kcount; ++kk) zeros_step(kk);
         } else {
             // some value of the k-tile needs the full definition: only the k-steps that hold one pay for it
-            uint32_t odd = 0u, zer = 0u;
+            uint32_t odd = 0u;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) { odd |= lds_odd_k[t & 1][w]; zer |= lds_zero_k[t & 1][w]; }
-            odd = __builtin_amdgcn_readfirstlane(odd); zer = __builtin_amdgcn_readfirstlane(zer);
+            for (int w = 0; w < NW; ++w) odd |= lds_odd_k[t & 1][w];
+            odd = __builtin_amdgcn_readfirstlane(odd);
+            const bool zeros = MODE == MODE_PAM && (verdict & (kZerosL | kZerosR)) != 0;    // somewhere in the tile
 #pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) {
                 if ((odd >> kk) & 1u) guarded_step(kk);
-                else if (MODE == MODE_PAM && ((zer >> kk) & 1u)) zeros_step(kk);
+                else if (zeros) zeros_step(kk);
                 else fast_step(kk);
             }
         }
