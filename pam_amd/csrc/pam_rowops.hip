@@ -447,6 +447,53 @@ __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], c
     }
 }
 
+// The all-exact gradient (the reference's default) without an offset, on unchecked arithmetic.  In the normal range
+// the exact backward formulas are short (pam/cuda_kernels.cu:40-58, 85-97, 115-123): the gradient of a (*) b for a
+// is g times 2^(exponent of b, plus one if the two fractions carry), i.e. the bits of b plus the fraction bits of a,
+// masked to sign and exponent; the quotient's gradient for its divisor is -(2^e(a (/) b) / 2^e(b)) g, a difference of
+// exponent fields; exp2's is 2^e(exp2 t) g.  The products with the upstream gradients are IEEE products in both
+// forms, so those gradients need no recording; everything else is recorded as in the approximate chain.
+template <int CH, class L>
+__device__ __forceinline__ void softmax_grad_row_exact(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
+                                                       float total, float shift, L& lay, long n, Unchecked& m)
+{
+    const uint32_t tot = f2u(total);
+    m.record(total);                                                       // a sum of weights: never negative
+    const uint32_t inv = kBias - tot + kBias;                              // 1 (/) total
+    m.sp.see(inv); m.sp.see(inv + 0x00800000u);                            // normal, and below 2^127 (a carry fits)
+    const uint32_t slope_c = f2u(kLog2E);
+    float e[CH];
+    float p = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool masked = f2u(xv[c]) == 0xff800000u;
+        const bool inside = lay.index(c) < n;
+        const float t = m.mul_const(masked ? 1.0f : xv[c], kLog2E) - shift;
+        e[c] = m.exp2(masked ? 0.5f : t);
+        // gradient of e (/) total for total: -(2^e(e (/) total) / 2^e(total)) g
+        const uint32_t quot = f2u(e[c]) - tot + kBias;                     // e (/) total, positive
+        const uint32_t ratio = (quot & kExpo) - (tot & kExpo) + kBias;
+        m.sp.see(quot); m.sp.see(ratio);
+        const float term = -u2f(ratio) * ((inside && !masked) ? g[c] : 1.0f);
+        // a masked element: e = 0, the quotient's gradient is -(0 / 2^e(total)) g, a zero for finite g and NaN otherwise
+        if (masked && inside) m.sp.see(f2u(g[c]) & ~kSign);
+        if (inside && !masked) p = p + term;
+    }
+    const float dtotal = lay.sum(p);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const bool masked = f2u(xv[c]) == 0xff800000u;
+        const bool inside = lay.index(c) < n;
+        const uint32_t ei = f2u(e[c]);
+        // e (/) total = e (*) inv for e: g 2^(e(inv) + carry)
+        const float de = ((inside && !masked) ? g[c] : 1.0f) * u2f((inv + (ei & kMant)) & ~kMant) + dtotal;
+        // exp2: 2^e(exp2 t) de; the product t (*) 1 in front of it passes its gradient on unchanged
+        const float dt = u2f(ei & ~kMant) * de;
+        // x (*) log2(e) for x
+        const float dx = dt * u2f((slope_c + (f2u(masked ? 1.0f : xv[c]) & kMant)) & ~kMant);
+        out[c] = masked ? 0.0f : dx;
+    }
+}
 // The same gradient with the checked primitives, for every combination of exact and approximate terms.
 template <int CH, class L, class AP>
 __device__ __forceinline__ void softmax_grad_row_checked_as(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
@@ -471,7 +518,9 @@ __device__ __forceinline__ void softmax_grad_row_checked(const float (&xv)[CH], 
     else softmax_grad_row_checked_as<CH>(xv, g, out, total, inv, shift, lay, n, o, ap);
 }
 
-template <int CH>
+// EXACT: the unchecked first attempt is the all-exact chain (chosen by the host for exact gradients without an offset);
+// otherwise it is the all-approximate one.  Every other combination goes to the checked functions directly.
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC_GRAD(CH)))) void softmax_bwd_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                               const float* __restrict__ row_sum, const float* __restrict__ shift_in,
                                                               float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
@@ -489,7 +538,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             load_row<CH>(g, gr, n, lane, 0.0f);
             bool done = false;
             WaveRow lay{lane};
-            if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient has an unchecked form
+            if (EXACT) {                                  // host: all exact, no offset
+                Unchecked u{o, Span()};
+                softmax_grad_row_exact<CH>(xv, g, out, total, shift, lay, n, u);
+                done = wave_valid(u);
+            } else if (ap.a && ap.b && ap.e) {            // the all-approximate gradient has an unchecked form
                 Unchecked u{o, Span()};
                 softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
                 done = wave_valid(u);
@@ -1076,7 +1129,7 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(C
     }
 }
 
-template <int CH>
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_bwd_block_kernel(const float* __restrict__ x, const float* __restrict__ dy,
                                                                          const float* __restrict__ row_sum, const float* __restrict__ shift_in,
                                                                          float* __restrict__ dx, long rows, long n, Offset o, Approx ap)
@@ -1089,7 +1142,11 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_bwd_bloc
         load_row<CH>(xv, x + r * n, n, lay, kNegInf);
         load_row<CH>(g, dy + r * n, n, lay, 0.0f);
         bool done = false;
-        if (ap.a && ap.b && ap.e) {
+        if (EXACT) {
+            Unchecked u{o, Span()};
+            softmax_grad_row_exact<CH>(xv, g, out, total, shift, lay, n, u);
+            done = lay.all(u.valid());
+        } else if (ap.a && ap.b && ap.e) {
             Unchecked u{o, Span()};
             softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
             done = lay.all(u.valid());
@@ -1223,6 +1280,15 @@ int block_chunks(long n)
 }
 bool block_rows(long n) { return n > kBlockRowMin && n <= kBlockRowMax; }
 
+#define PAM_BLOCK_DISPATCH_FLAG(KERNEL, FLAG, n, grid, st, ...)                                                 \
+    switch (block_chunks(n)) {                                                                                  \
+    case 6: hipLaunchKernelGGL((KERNEL<6, FLAG>), grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;        \
+    case 8: hipLaunchKernelGGL((KERNEL<8, FLAG>), grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;        \
+    case 10: hipLaunchKernelGGL((KERNEL<10, FLAG>), grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;      \
+    case 12: hipLaunchKernelGGL((KERNEL<12, FLAG>), grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;      \
+    default: hipLaunchKernelGGL((KERNEL<16, FLAG>), grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;      \
+    }
+
 #define PAM_BLOCK_DISPATCH(KERNEL, n, grid, st, ...)                                                            \
     switch (block_chunks(n)) {                                                                                  \
     case 6: hipLaunchKernelGGL(KERNEL<6>, grid, dim3(kBlockThreads), 0, st, __VA_ARGS__); break;                \
@@ -1247,6 +1313,16 @@ int row_chunks(long n)
     case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 16: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     default: hipLaunchKernelGGL(KERNEL<0>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                    \
+    }
+
+#define PAM_ROW_DISPATCH_FLAG(KERNEL, FLAG, n, grid, st, ...)                                                   \
+    switch (row_chunks(n)) {                                                                                    \
+    case 1: hipLaunchKernelGGL((KERNEL<1, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 2: hipLaunchKernelGGL((KERNEL<2, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 4: hipLaunchKernelGGL((KERNEL<4, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 8: hipLaunchKernelGGL((KERNEL<8, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 16: hipLaunchKernelGGL((KERNEL<16, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;           \
+    default: hipLaunchKernelGGL((KERNEL<0, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;            \
     }
 
 #define PAM_ROW_DISPATCH_REGS(KERNEL, n, grid, st, ...)                                                         \
@@ -1347,10 +1423,13 @@ int pam_hip_softmax_bwd(const float* x, const float* dy, const float* row_sum, c
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !dy || !row_sum || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "softmax_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
+    const bool exact_fast = !ap.a && !ap.b && !ap.e && !o.has;
     if (block_rows(n)) {
-        PAM_BLOCK_DISPATCH(softmax_bwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap);
+        if (exact_fast) { PAM_BLOCK_DISPATCH_FLAG(softmax_bwd_block_kernel, true, n, dim3(block_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap); }
+        else { PAM_BLOCK_DISPATCH_FLAG(softmax_bwd_block_kernel, false, n, dim3(block_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap); }
     } else {
-        PAM_ROW_DISPATCH(softmax_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap);
+        if (exact_fast) { PAM_ROW_DISPATCH_FLAG(softmax_bwd_kernel, true, n, dim3(row_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap); }
+        else { PAM_ROW_DISPATCH_FLAG(softmax_bwd_kernel, false, n, dim3(row_grid(rows)), (hipStream_t)stream, x, dy, row_sum, shift, dx, rows, n, o, ap); }
     }
     return pamhost::check_launch("softmax_bwd");
 }
