@@ -270,6 +270,8 @@ def main():
             )
             row_ops += (("log_softmax_bwd_approx", 12, lambda: R.logsumexp_bwd(xs, gs, sh, 1.0, True, True, True, True)),)
             row_ops += (("layer_norm_bwd_approx", 16, lambda: R.layer_norm_bwd(xs, wv, gs, 1e-5, 1.0, True, True, True, True)),)
+            row_ops += (("log_softmax_bwd_exact", 12, lambda: R.logsumexp_bwd(xs, gs, sh, 1.0, False, False, False, True)),)
+            row_ops += (("layer_norm_bwd_exact", 16, lambda: R.layer_norm_bwd(xs, wv, gs, 1e-5, 1.0, False, False, False, True)),)
             for name, bpe, fn in row_ops:
                 ms = event_time_ms(fn, 30, torch)
                 other[f"{name}_{tag}"] = {"ms": round(ms, 4), "GBps": round(bpe * r * c / ms / 1e6, 1),

@@ -19,6 +19,7 @@
 #include <math.h>
 
 #include <atomic>
+#include <type_traits>
 
 #include "pam_common.h"
 #include "pam_device.h"
@@ -779,6 +780,43 @@ struct GradUnchecked {
     __device__ __forceinline__ bool valid() const { return sp.normal(); }
 };
 
+// The all-exact gradients (the reference's default) without an offset, on unchecked arithmetic.  In the normal range
+// the exact backward formulas are short (pam/cuda_kernels.cu:40-58, 85-97, 115-123, 132-136): the gradient of a (*) b
+// for a is g 2^(e(b) + carry of the two fractions) with b's sign, i.e. the bits of b plus the fraction bits of a masked
+// to sign and exponent; of a (/) b for b, -(2^e(a (/) b) / 2^e(b)) g, a difference of exponent fields; of exp2,
+// 2^e(exp2 x) g; of log2, 2^-e(x) g.  The products with the upstream gradients are IEEE products in the checked forms
+// too, so the gradients need no recording; the other operands are recorded, with the extra headroom the carries need.
+struct GradUncheckedExact {
+    Offset o; Span sp;                            // used without an offset only
+    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked(a, b, sp); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked(a, b, sp); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, 1.0f, false, sp); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, 1.0f, false, sp); }
+    __device__ __forceinline__ float mul_da(float a, float b, float g)
+    {
+        const uint32_t ai = f2u(a), bi = f2u(b), mb = bi & ~kSign;
+        sp.see(ai & ~kSign); sp.see(mb); sp.see(mb + 0x00800000u);             // b below 2^127: the carry fits
+        return g * u2f((bi + (ai & kMant)) & ~kMant);
+    }
+    __device__ __forceinline__ float mul_db(float a, float b, float g) { return mul_da(b, a, g); }
+    __device__ __forceinline__ float div_da(float a, float b, float g) { return mul_da(a, div(1.0f, b), g); }
+    __device__ __forceinline__ float div_db(float a, float b, float g)
+    {
+        const uint32_t oi = f2u(div(a, b));
+        const uint32_t ratio = (oi & kExpo) - (f2u(b) & kExpo) + kBias;        // a wrap lands above the exponent mask and is caught
+        sp.see(ratio);
+        return -u2f(ratio | (oi & kSign)) * g;
+    }
+    __device__ __forceinline__ float exp2_dx(float x, float g) { return u2f(f2u(exp2(x)) & ~kMant) * g; }
+    __device__ __forceinline__ float log2_dx(float x, float g)
+    {
+        const uint32_t xi = f2u(x);                                            // positive (a sign bit reads as too large), below 2^127
+        sp.see(xi); sp.see(xi + 0x00800000u);
+        return u2f((254u << 23) - (xi & kExpo)) * g;
+    }
+    __device__ __forceinline__ bool valid() const { return sp.normal(); }
+};
+
 // One row of the logsumexp / log_softmax gradient.  xv: the inputs (any fill past the end); gy: the
 // per-element gradients (log_softmax) with 1.0 past the end; out: dx.  Lanes past the end of the
 // row work on stand-in values that are never stored or summed.
@@ -809,7 +847,7 @@ __device__ __forceinline__ void logsumexp_grad_row(const float (&xv)[CH], const 
 }
 
 // dx of out = logsumexp(x) (per row, gradient g_out) or of y = x - logsumexp(x) (gradient gy per element)
-template <int CH>
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_OCC_GRAD(CH)))) void logsumexp_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
     long rows, long n, int log_softmax, Offset o, Approx ap)
@@ -826,8 +864,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
         WaveRow lay{lane};
-        if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o, Span()};
+        if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
+            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
             logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -886,6 +924,7 @@ __device__ __forceinline__ void logsumexp_grad_stream(const float* __restrict__ 
     }
 }
 
+template <bool EXACT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void logsumexp_bwd_stream_kernel(
     const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
     long rows, long n, int log_softmax, Offset o, Approx ap)
@@ -897,8 +936,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         const float* gr = log_softmax ? grad + r * n : nullptr;
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
-        if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o, Span()};
+        if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
+            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
             logsumexp_grad_stream(x + r * n, gr, dx + r * n, g_row, log_softmax != 0, shift, lane, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1022,6 +1061,7 @@ __device__ __forceinline__ void layer_norm_grad_stream(const float* __restrict__
     for (int i = lane; i < n; i += 64) dr[i] = dr[i] + ds1;
 }
 
+template <bool EXACT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_ROW_WAVES))) void layer_norm_bwd_stream_kernel(
     const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
     float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
@@ -1032,8 +1072,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     for (long r = wave; r < rows; r += nwaves) {
         float* tr = (weight && dw_terms) ? dw_terms + r * n : nullptr;
         bool done = false;
-        if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o, Span()};
+        if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
+            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
             layer_norm_grad_stream(x + r * n, gy + r * n, weight, dx + r * n, tr, lane, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1043,7 +1083,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 
 // dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias.  Rows of 1024 values: three
 // wavefronts per SIMD (168 registers); left at two the compiler takes 181 and a third fewer wavefronts fit.
-template <int CH>
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >= 16 ? 3 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
     float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
@@ -1055,10 +1095,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >
         float cen[CH], g[CH], terms[CH];
         bool done = false;
         WaveRow lay{lane};
-        if (ap.a && ap.b && ap.e) {
+        if (EXACT || (ap.a && ap.b && ap.e)) {
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
-            GradUnchecked u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
             layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1219,7 +1259,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_fwd_b
     }
 }
 
-template <int CH>
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_bwd_block_kernel(
     const float* __restrict__ x, const float* __restrict__ grad, const float* __restrict__ shift_in, float* __restrict__ dx,
     long rows, long n, int log_softmax, Offset o, Approx ap)
@@ -1234,8 +1274,8 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_bwd_bl
         if (log_softmax) load_row<CH>(gy, grad + r * n, n, lay, 1.0f);
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
-        if (ap.a && ap.b && ap.e) {
-            GradUnchecked u{o, Span()};
+        if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
+            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
             logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, u);
             done = lay.all(u.valid());
         }
@@ -1244,7 +1284,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_bwd_bl
     }
 }
 
-template <int CH>
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_bwd_block_kernel(
     const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
     float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
@@ -1254,10 +1294,10 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_bwd_b
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float cen[CH], g[CH], terms[CH];
         bool done = false;
-        if (ap.a && ap.b && ap.e) {
+        if (EXACT || (ap.a && ap.b && ap.e)) {
             load_row<CH>(cen, x + r * n, n, lay, 0.0f);
             load_row<CH>(g, gy + r * n, n, lay, 1.0f);
-            GradUnchecked u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
             layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, u);
             done = lay.all(u.valid());
         }
@@ -1323,6 +1363,15 @@ int row_chunks(long n)
     case 8: hipLaunchKernelGGL((KERNEL<8, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 16: hipLaunchKernelGGL((KERNEL<16, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;           \
     default: hipLaunchKernelGGL((KERNEL<0, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;            \
+    }
+
+#define PAM_ROW_DISPATCH_REGS_FLAG(KERNEL, FLAG, n, grid, st, ...)                                              \
+    switch (row_chunks(n)) {                                                                                    \
+    case 1: hipLaunchKernelGGL((KERNEL<1, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 2: hipLaunchKernelGGL((KERNEL<2, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 4: hipLaunchKernelGGL((KERNEL<4, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 8: hipLaunchKernelGGL((KERNEL<8, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    default: hipLaunchKernelGGL((KERNEL<16, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;           \
     }
 
 #define PAM_ROW_DISPATCH_REGS(KERNEL, n, grid, st, ...)                                                         \
@@ -1493,15 +1542,20 @@ int pam_hip_logsumexp_bwd(const float* x, const float* grad, const float* shift,
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !grad || !shift || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "logsumexp_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    if (block_rows(n)) {
-        PAM_BLOCK_DISPATCH(logsumexp_bwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n,
-                           log_softmax, o, ap);
-    } else if (n > 1024)
-        hipLaunchKernelGGL(logsumexp_bwd_stream_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, grad, shift, dx,
-                           rows, n, log_softmax, o, ap);
-    else
-        PAM_ROW_DISPATCH_REGS(logsumexp_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n,
-                              log_softmax, o, ap);
+    const bool exact_fast = !ap.a && !ap.b && !ap.e && !o.has;
+#define PAM_LSE_BWD(FLAG)                                                                                                       \
+    if (block_rows(n)) {                                                                                                        \
+        PAM_BLOCK_DISPATCH_FLAG(logsumexp_bwd_block_kernel, FLAG, n, dim3(block_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n, \
+                                log_softmax, o, ap);                                                                            \
+    } else if (n > 1024)                                                                                                        \
+        hipLaunchKernelGGL(logsumexp_bwd_stream_kernel<FLAG>, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, grad, shift, dx, \
+                           rows, n, log_softmax, o, ap);                                                                        \
+    else {                                                                                                                      \
+        PAM_ROW_DISPATCH_REGS_FLAG(logsumexp_bwd_kernel, FLAG, n, dim3(row_grid(rows)), (hipStream_t)stream, x, grad, shift, dx, rows, n, \
+                                   log_softmax, o, ap);                                                                         \
+    }
+    if (exact_fast) { PAM_LSE_BWD(true) } else { PAM_LSE_BWD(false) }
+#undef PAM_LSE_BWD
     return pamhost::check_launch("logsumexp_bwd");
 }
 
@@ -1513,15 +1567,20 @@ int pam_hip_layer_norm_bwd(const float* x, const float* weight, const float* dy,
     if (rows == 0 || n == 0) return PAM_HIP_OK;
     if (!x || !dy || !dx) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "layer_norm_bwd: null pointer");
     Offset o{offset, offset != 1.0f}; Approx ap{approx_a != 0, approx_b != 0, approx_exp != 0};
-    if (block_rows(n)) {
-        PAM_BLOCK_DISPATCH(layer_norm_bwd_block_kernel, n, dim3(block_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms,
-                           rows, n, eps, o, ap);
-    } else if (n > 1024)
-        hipLaunchKernelGGL(layer_norm_bwd_stream_kernel, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, weight, dy, dx,
-                           dw_terms, rows, n, eps, o, ap);
-    else
-        PAM_ROW_DISPATCH_REGS(layer_norm_bwd_kernel, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms,
-                              rows, n, eps, o, ap);
+    const bool exact_fast = !ap.a && !ap.b && !ap.e && !o.has;
+#define PAM_LN_BWD(FLAG)                                                                                                        \
+    if (block_rows(n)) {                                                                                                        \
+        PAM_BLOCK_DISPATCH_FLAG(layer_norm_bwd_block_kernel, FLAG, n, dim3(block_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms, \
+                                rows, n, eps, o, ap);                                                                           \
+    } else if (n > 1024)                                                                                                        \
+        hipLaunchKernelGGL(layer_norm_bwd_stream_kernel<FLAG>, dim3(row_grid(rows)), dim3(kThreads), 0, (hipStream_t)stream, x, weight, dy, dx, \
+                           dw_terms, rows, n, eps, o, ap);                                                                      \
+    else {                                                                                                                      \
+        PAM_ROW_DISPATCH_REGS_FLAG(layer_norm_bwd_kernel, FLAG, n, dim3(row_grid(rows)), (hipStream_t)stream, x, weight, dy, dx, dw_terms, \
+                                   rows, n, eps, o, ap);                                                                        \
+    }
+    if (exact_fast) { PAM_LN_BWD(true) } else { PAM_LN_BWD(false) }
+#undef PAM_LN_BWD
     return pamhost::check_launch("layer_norm_bwd");
 }
 

@@ -307,10 +307,48 @@ def test_gpu_softmax_special_values(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("n", [100, 700, 2000])
+def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n):
+    """All-exact gradients without an offset first run on unchecked arithmetic: inputs and upstream gradients at and
+    beyond the edges of what that accepts (zeros, subnormals, huge and tiny values, inf, NaN, a variance of exactly 1)."""
+    rng = np.random.RandomState(n)
+    x = (rng.standard_normal((12, n)) * 3).astype(np.float32)
+    x[1, 3] = 0.0; x[2, 5] = 1e-40; x[3, 7] = 3e38; x[4, 9] = -3e38; x[5, 11] = 2.0 ** -120; x[6, :] = 2.0 ** 100; x[7, 13] = -np.inf
+    x[8, :] = np.where(np.arange(n) % 2 == 0, 1.0, -1.0)             # mean 0, variance 1 (n even)
+    g = rng.standard_normal(x.shape).astype(np.float32)
+    g[0, 1] = 0.0; g[0, 2] = 1e-42; g[1, 4] = np.inf; g[2, 6] = np.nan; g[3, 8] = 3e38; g[9, :] = 0.0; g[10, 3] = 2.0 ** -130
+    flags = (False, False, False)
+    xt = _dev(x).requires_grad_()
+    y = pam_amd.softmax(xt, dim=-1)
+    want, row_sum, shift = oracle.softmax_fwd(x)
+    assert_same_bits(y.detach().cpu().numpy(), want, "softmax")
+    y.backward(_dev(g))
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, None, flags), "softmax gradient")
+    xf = np.where(np.isfinite(x), x, np.float32(1.5)).astype(np.float32)
+    xt = _dev(xf).requires_grad_()
+    y = pam_amd.log_softmax(xt, dim=-1)
+    y.backward(_dev(g))
+    sh = np.floor(oracle.pam(xf, C).max())
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g, sh, None, flags, log_softmax=True), "log_softmax gradient")
+    xt = _dev(xf).requires_grad_()
+    pam_amd.logsumexp(xt, dim=-1).backward(_dev(g[:, 0].copy()))
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g[:, 0].copy(), sh, None, flags), "logsumexp gradient")
+    w = (rng.standard_normal(n) + 2).astype(np.float32); w[3] = 0.0; w[5] = 1e-39; w[7] = -2.0
+    for ww in (None, w):
+        xt = _dev(xf).requires_grad_()
+        wt = None if ww is None else _dev(ww).requires_grad_()
+        y = pam_amd.layer_norm(xt, n, wt, None)
+        y.backward(_dev(g))
+        dx, _ = oracle.layer_norm_bwd(xf, ww, g, 1e-5, None, flags)
+        assert_same_bits(xt.grad.cpu().numpy(), dx, "layer_norm gradient")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("approx", [True, False])
 @pytest.mark.parametrize("off", [None, OFF])
-def test_gpu_long_rows_with_special_values(oracle, off):
+def test_gpu_long_rows_with_special_values(oracle, off, approx):
     """Rows held by a whole work-group: a value outside the normal range anywhere in the row sends every
-    thread of the row to the checked arithmetic (forward and all-approximate gradients)."""
+    thread of the row to the checked arithmetic (forward, all-approximate and all-exact gradients)."""
     n = 9000
     x = rows_case(77, 6, n, masks=False)
     x[1, 8999] = 0.0; x[2, 1024] = 1e-40; x[3, 5000] = np.inf; x[4, 63] = -np.inf; x[5, 4000] = np.nan
@@ -318,25 +356,25 @@ def test_gpu_long_rows_with_special_values(oracle, off):
     g[0, 77] = 0.0; g[1, 5] = 1e-41
     w = (np.random.RandomState(9).standard_normal(n) + 2).astype(np.float32); w[17] = 0.0
     xt = _dev(x).requires_grad_()
-    y = pam_amd.softmax(xt, dim=-1, offset=off, approx_bwd=True)
+    y = pam_amd.softmax(xt, dim=-1, offset=off, approx_bwd=approx)
     want, row_sum, shift = oracle.softmax_fwd(x, off)
     assert_same_bits(y.detach().cpu().numpy(), want, "softmax")
     y.backward(_dev(g))
-    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, off, (True, True, True)), "softmax gradient")
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, off, (approx, approx, approx)), "softmax gradient")
     xs = x[:3]                                       # finite rows for the shifted ops
     lse, ls = oracle.logsumexp_fwd(xs, off, with_log_softmax=True)
     xt = _dev(xs).requires_grad_()
-    y = pam_amd.log_softmax(xt, dim=-1, offset=off, approx_bwd=True)
+    y = pam_amd.log_softmax(xt, dim=-1, offset=off, approx_bwd=approx)
     assert_same_bits(y.detach().cpu().numpy(), ls, "log_softmax")
     y.backward(_dev(g[:3]))
     sh = np.floor(oracle.pam(xs, C, off).max())
-    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xs, g[:3], sh, off, (True, True, True), log_softmax=True), "log_softmax gradient")
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xs, g[:3], sh, off, (approx, approx, approx), log_softmax=True), "log_softmax gradient")
     assert_same_bits(pam_amd.mean(_dev(x), dim=-1, offset=off).cpu().numpy(), oracle.row_mean_fwd(x, off), "mean")
     xt = _dev(x).requires_grad_(); wt = _dev(w).requires_grad_()
-    y = pam_amd.layer_norm(xt, n, wt, None, offset=off, approx_bwd=True)
+    y = pam_amd.layer_norm(xt, n, wt, None, offset=off, approx_bwd=approx)
     assert_same_bits(y.detach().cpu().numpy(), oracle.layer_norm_fwd(x, w, None, 1e-5, off), "layer_norm")
     y.backward(_dev(g))
-    dx, _ = oracle.layer_norm_bwd(x, w, g, 1e-5, off, (True, True, True))
+    dx, _ = oracle.layer_norm_bwd(x, w, g, 1e-5, off, (approx, approx, approx))
     assert_same_bits(xt.grad.cpu().numpy(), dx, "layer_norm gradient")
 
 
