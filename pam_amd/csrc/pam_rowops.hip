@@ -553,7 +553,32 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) dr[i] = out[c]; }
         } else {
             bool done = false;
-            if (ap.a && ap.b && ap.e) {                   // the all-approximate gradient, branch-free forms first
+            if (EXACT) {                                  // the all-exact gradient as in softmax_grad_row_exact, in two sweeps
+                Unchecked m{o, Span()};
+                const uint32_t tot = f2u(total), inv_b = kBias - tot + kBias, slope_c = f2u(kLog2E);
+                m.record(total); m.sp.see(inv_b); m.sp.see(inv_b + 0x00800000u);
+                auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul_const(masked ? 1.0f : x, kLog2E) - shift); };
+                float p = 0.0f;
+                for_blocks2(xr, gr, (int)n, lane, kNegInf, 1.0f, [&](long, bool inside, float x, float gi) {
+                    const bool masked = f2u(x) == 0xff800000u;
+                    const uint32_t quot = f2u(weight(x, masked)) - tot + kBias;
+                    const uint32_t ratio = (quot & kExpo) - (tot & kExpo) + kBias;
+                    m.sp.see(quot); m.sp.see(ratio);
+                    const float term = -u2f(ratio) * (masked ? 1.0f : gi);
+                    if (masked && inside) m.sp.see(f2u(gi) & ~kSign);
+                    if (inside && !masked) p = p + term;
+                });
+                const float dtotal = wave_sum(p);
+                for_blocks2(xr, gr, (int)n, lane, kNegInf, 1.0f, [&](long i, bool inside, float x, float gi) {
+                    const bool masked = f2u(x) == 0xff800000u;
+                    const uint32_t ei = f2u(weight(x, masked));
+                    const float de = (masked ? 1.0f : gi) * u2f((inv_b + (ei & kMant)) & ~kMant) + dtotal;
+                    const float dt = u2f(ei & ~kMant) * de;
+                    const float d = dt * u2f((slope_c + (f2u(masked ? 1.0f : x) & kMant)) & ~kMant);
+                    if (inside) dr[i] = masked ? 0.0f : d;
+                });
+                done = wave_valid(m);
+            } else if (ap.a && ap.b && ap.e) {            // the all-approximate gradient, branch-free forms first
                 Unchecked m{o, Span()};
                 const float inv_u = m.div(1.0f, total);
                 auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
