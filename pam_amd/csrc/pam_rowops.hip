@@ -1106,10 +1106,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     }
 }
 
-// dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias.  Rows of 1024 values: three
-// wavefronts per SIMD (168 registers); left at two the compiler takes 181 and a third fewer wavefronts fit.
+// dx and the per-element weight-gradient terms of y = layer_norm(x) * weight + bias.  Rows of 1024 values (and of 768
+// for the exact chain, by measurement): three wavefronts per SIMD (168 registers); left at two the compiler takes 181
+// and a third fewer wavefronts fit.
 template <int CH, bool EXACT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((CH) >= 16 ? 3 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(((CH) >= 16 || ((CH) >= 12 && EXACT)) ? 3 : ((CH) <= 4 ? 6 : PAM_ROW_WAVES)))) void layer_norm_bwd_kernel(
     const float* __restrict__ x, const float* __restrict__ weight, const float* __restrict__ gy, float* __restrict__ dx,
     float* __restrict__ dw_terms, long rows, long n, float eps, Offset o, Approx ap)
 {
@@ -1366,7 +1367,7 @@ bool block_rows(long n) { return n > kBlockRowMin && n <= kBlockRowMax; }
 // smallest register-resident variant that holds a row of n values, 0 for the streaming one
 int row_chunks(long n)
 {
-    for (int ch : {1, 2, 4, 8, 16}) if (n <= 64L * ch) return ch;
+    for (int ch : {1, 2, 3, 4, 6, 8, 12, 16}) if (n <= 64L * ch) return ch;          // 3, 6, 12: rows of 192, 384, 768 values
     return 0;
 }
 
@@ -1374,8 +1375,11 @@ int row_chunks(long n)
     switch (row_chunks(n)) {                                                                                    \
     case 1: hipLaunchKernelGGL(KERNEL<1>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 2: hipLaunchKernelGGL(KERNEL<2>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 3: hipLaunchKernelGGL(KERNEL<3>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 4: hipLaunchKernelGGL(KERNEL<4>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 6: hipLaunchKernelGGL(KERNEL<6>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 12: hipLaunchKernelGGL(KERNEL<12>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     case 16: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     default: hipLaunchKernelGGL(KERNEL<0>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                    \
     }
@@ -1384,8 +1388,11 @@ int row_chunks(long n)
     switch (row_chunks(n)) {                                                                                    \
     case 1: hipLaunchKernelGGL((KERNEL<1, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 2: hipLaunchKernelGGL((KERNEL<2, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 3: hipLaunchKernelGGL((KERNEL<3, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 4: hipLaunchKernelGGL((KERNEL<4, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 6: hipLaunchKernelGGL((KERNEL<6, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 8: hipLaunchKernelGGL((KERNEL<8, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 12: hipLaunchKernelGGL((KERNEL<12, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 16: hipLaunchKernelGGL((KERNEL<16, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;           \
     default: hipLaunchKernelGGL((KERNEL<0, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;            \
     }
@@ -1394,8 +1401,11 @@ int row_chunks(long n)
     switch (row_chunks(n)) {                                                                                    \
     case 1: hipLaunchKernelGGL((KERNEL<1, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 2: hipLaunchKernelGGL((KERNEL<2, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 3: hipLaunchKernelGGL((KERNEL<3, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 4: hipLaunchKernelGGL((KERNEL<4, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 6: hipLaunchKernelGGL((KERNEL<6, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     case 8: hipLaunchKernelGGL((KERNEL<8, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
+    case 12: hipLaunchKernelGGL((KERNEL<12, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;             \
     default: hipLaunchKernelGGL((KERNEL<16, FLAG>), grid, dim3(kThreads), 0, st, __VA_ARGS__); break;           \
     }
 
@@ -1403,8 +1413,11 @@ int row_chunks(long n)
     switch (row_chunks(n)) {                                                                                    \
     case 1: hipLaunchKernelGGL(KERNEL<1>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 2: hipLaunchKernelGGL(KERNEL<2>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 3: hipLaunchKernelGGL(KERNEL<3>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 4: hipLaunchKernelGGL(KERNEL<4>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 6: hipLaunchKernelGGL(KERNEL<6>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
     case 8: hipLaunchKernelGGL(KERNEL<8>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                     \
+    case 12: hipLaunchKernelGGL(KERNEL<12>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     default: hipLaunchKernelGGL(KERNEL<16>, grid, dim3(kThreads), 0, st, __VA_ARGS__); break;                   \
     }
 

@@ -254,7 +254,7 @@ def _dev(a):
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_softmax_forward_backward(oracle, off):
     # 4097 ... 16384 values: a work-group per row
-    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (64, 197), (2, 1000), (300, 32), (3, 4096), (5, 4097), (3, 6145), (2, 10000),
+    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (64, 197), (7, 300), (7, 384), (2, 1000), (300, 32), (3, 4096), (5, 4097), (3, 6145), (2, 10000),
                     (2, 16384), (2, 16385)]:
         x = rows_case(rows * 1000 + n, rows, n)
         g = np.random.RandomState(n).standard_normal(x.shape).astype(np.float32)
@@ -412,7 +412,7 @@ def test_gpu_more_rows_than_the_launch_holds(oracle, rows, n):
 @pytest.mark.gpu
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_logsumexp_mean_layer_norm(oracle, off):
-    for rows, n in [(1, 1), (3, 7), (4, 64), (50, 192), (2, 513), (33, 512), (2, 4096), (3, 4097), (3, 8193), (3, 10000), (2, 12289), (2, 16384), (2, 16385)]:
+    for rows, n in [(1, 1), (3, 7), (4, 64), (50, 192), (5, 384), (2, 513), (33, 512), (3, 768), (2, 4096), (3, 4097), (3, 8193), (3, 10000), (2, 12289), (2, 16384), (2, 16385)]:
         x = rows_case(rows * 77 + n, rows, n, masks=False)
         xt = _dev(x)
         lse, ls = oracle.logsumexp_fwd(x, off, with_log_softmax=True)
@@ -462,7 +462,7 @@ def test_gpu_attention_softmax_full_size(oracle):
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_logsumexp_and_layer_norm_gradients(oracle, off):
     # rows beyond 1024 values: the gradient kernels sweep the row several times instead of holding it in registers
-    for rows, n in [(1, 1), (3, 7), (5, 64), (40, 192), (9, 513), (6, 1024), (5, 1025), (3, 2500), (2, 4097), (2, 6200), (2, 10000), (2, 12300), (2, 16384), (2, 16385)]:
+    for rows, n in [(1, 1), (3, 7), (5, 64), (40, 192), (6, 384), (9, 513), (4, 768), (6, 1024), (5, 1025), (3, 2500), (2, 4097), (2, 6200), (2, 10000), (2, 12300), (2, 16384), (2, 16385)]:
         x = rows_case(rows * 13 + n, rows, n, masks=False)
         rng = np.random.RandomState(n)
         g_rows = rng.standard_normal(rows).astype(np.float32); g_full = rng.standard_normal(x.shape).astype(np.float32)
