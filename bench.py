@@ -255,7 +255,8 @@ def main():
         # row-wise compositions as single kernels and the Adam step (HBM-bound; algorithmic bytes per element)
         from pam_amd import _abi as abi
         R = abi.HipRowKernels()
-        rows_cases = {"attention_37824x197": (192 * 197, 197), "rows_65536x1024": (65536, 1024), "vocabulary_4096x10000": (4096, 10000)}
+        rows_cases = {"attention_37824x197": (192 * 197, 197), "rows_65536x1024": (65536, 1024), "vocabulary_4096x10000": (4096, 10000),
+                      "deit_tiny_tokens_50432x192": (256 * 197, 192)}     # the layer_norm shape of the headline model (256 images)
         for tag, (r, c) in rows_cases.items():
             xs = torch.randn(r, c, generator=g).to(dev); gs = torch.randn(r, c, generator=g).to(dev)
             wv = torch.randn(c, generator=g).to(dev); bv = torch.randn(c, generator=g).to(dev)
