@@ -359,27 +359,47 @@ typedef const __attribute__((address_space(3))) u32x4* LdsVec;
 // of the next product issued ahead of the float add of the current one.  Written out because the compiler, given
 // the unrolled k-tile as one block, moves all of its LDS reads to the top and spills; the LDS addresses pass
 // through (unchanged) so that the reads of the step after next cannot be issued before this block.
-__device__ __forceinline__ void pam_mac_4x4(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
-{
-    uint32_t t0, t1;
+#define PAM_ACC_OPERANDS                                                                                      \
+    [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),               \
+    [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),               \
+    [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),               \
+    [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3])
+#define PAM_FRAGMENT_OPERANDS \
+    [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w)
 #define PAM_MAC_ROW(I)                                              \
     "v_add_u32 %[t1], %[a" #I "], %[b1]\n v_add_f32 %[c" #I "0], %[c" #I "0], %[t0]\n" \
     "v_add_u32 %[t0], %[a" #I "], %[b2]\n v_add_f32 %[c" #I "1], %[c" #I "1], %[t1]\n" \
     "v_add_u32 %[t1], %[a" #I "], %[b3]\n v_add_f32 %[c" #I "2], %[c" #I "2], %[t0]\n"
-    asm volatile(
-        "v_add_u32 %[t0], %[a0], %[b0]\n"
-        PAM_MAC_ROW(0) "v_add_u32 %[t0], %[a1], %[b0]\n v_add_f32 %[c03], %[c03], %[t1]\n"
-        PAM_MAC_ROW(1) "v_add_u32 %[t0], %[a2], %[b0]\n v_add_f32 %[c13], %[c13], %[t1]\n"
-        PAM_MAC_ROW(2) "v_add_u32 %[t0], %[a3], %[b0]\n v_add_f32 %[c23], %[c23], %[t1]\n"
-        PAM_MAC_ROW(3) "v_add_f32 %[c33], %[c33], %[t1]\n"
-        : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),
-          [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
-          [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),
-          [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
-          [t0] "=&v"(t0), [t1] "=&v"(t1), [pl] "+v"(pl), [pr] "+v"(pr)
-        : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
-#undef PAM_MAC_ROW
+#define PAM_MAC_BODY                                                                  \
+    "v_add_u32 %[t0], %[a0], %[b0]\n"                                                 \
+    PAM_MAC_ROW(0) "v_add_u32 %[t0], %[a1], %[b0]\n v_add_f32 %[c03], %[c03], %[t1]\n" \
+    PAM_MAC_ROW(1) "v_add_u32 %[t0], %[a2], %[b0]\n v_add_f32 %[c13], %[c13], %[t1]\n" \
+    PAM_MAC_ROW(2) "v_add_u32 %[t0], %[a3], %[b0]\n v_add_f32 %[c23], %[c23], %[t1]\n" \
+    PAM_MAC_ROW(3) "v_add_f32 %[c33], %[c33], %[t1]\n"
+__device__ __forceinline__ void pam_mac_4x4(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
+{
+    uint32_t t0, t1;
+    asm volatile(PAM_MAC_BODY
+                 : PAM_ACC_OPERANDS, [t0] "=&v"(t0), [t1] "=&v"(t1), [pl] "+v"(pl), [pr] "+v"(pr)
+                 : PAM_FRAGMENT_OPERANDS);
 }
+
+// The same block under a wavefront-uniform lane mask `run` (all ones or zero): with zero the instructions issue and
+// change nothing.  For a loop whose k-steps are of two kinds, so that the accumulators pass through the same
+// statement in every step and keep their registers (a branch around the statement made the compiler copy all sixteen
+// before and after it).
+__device__ __forceinline__ void pam_mac_4x4_under(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr,
+                                                  uint64_t run)
+{
+    uint32_t t0, t1;
+    uint64_t all;
+    asm volatile("s_mov_b64 %[all], exec\n s_and_b64 exec, exec, %[run]\n" PAM_MAC_BODY "s_mov_b64 exec, %[all]\n"
+                 : PAM_ACC_OPERANDS, [t0] "=&v"(t0), [t1] "=&v"(t1), [all] "=&s"(all), [pl] "+v"(pl), [pr] "+v"(pr)
+                 : PAM_FRAGMENT_OPERANDS, [run] "s"(run)
+                 : "scc");
+}
+#undef PAM_MAC_BODY
+#undef PAM_MAC_ROW
 
 // The same sixteen products for a k-tile whose LEFT (else right) operand holds zeros next to in-range values.  A PAM
 // product with a zero is +0 and adding it changes nothing (the sums start at +0 and never become -0), so those
@@ -434,71 +454,114 @@ __device__ __forceinline__ void pam_mac_4x4_skip(float (&acc)[4][4], const u32x4
 // Zeros in both operands: a product runs in the lanes where neither value is the staged zero.  Eight compares give
 // the masks of the four left and four right values, the integer sums of a row are formed in all lanes, and each
 // float add runs under the AND of its two masks (formed on the scalar unit).
-__device__ __forceinline__ void pam_mac_4x4_skip_both(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
-{
-    uint32_t t0, t1, t2, t3;
-    uint64_t all, ma0, ma1, ma2, ma3, mb0, mb1, mb2, mb3;
-#define PAM_BOTH_ROW(I)                                                                         \
-    "s_mov_b64 exec, %[all]\n"                                                                  \
+#define PAM_BOTH_ROW(I, LIVE)                                                                   \
+    "s_mov_b64 exec, %[" LIVE "]\n"                                                             \
     "v_add_u32 %[t0], %[a" #I "], %[b0]\n v_add_u32 %[t1], %[a" #I "], %[b1]\n"                  \
     "v_add_u32 %[t2], %[a" #I "], %[b2]\n v_add_u32 %[t3], %[a" #I "], %[b3]\n"                  \
     "s_and_b64 exec, %[ma" #I "], %[mb0]\n v_add_f32 %[c" #I "0], %[c" #I "0], %[t0]\n"          \
     "s_and_b64 exec, %[ma" #I "], %[mb1]\n v_add_f32 %[c" #I "1], %[c" #I "1], %[t1]\n"          \
     "s_and_b64 exec, %[ma" #I "], %[mb2]\n v_add_f32 %[c" #I "2], %[c" #I "2], %[t2]\n"          \
     "s_and_b64 exec, %[ma" #I "], %[mb3]\n v_add_f32 %[c" #I "3], %[c" #I "3], %[t3]\n"
+#define PAM_BOTH_MASKS                                                                          \
+    "v_cmp_ne_u32_e64 %[ma0], 0, %[a0]\n v_cmp_ne_u32_e64 %[ma1], 0, %[a1]\n"                    \
+    "v_cmp_ne_u32_e64 %[ma2], 0, %[a2]\n v_cmp_ne_u32_e64 %[ma3], 0, %[a3]\n"                    \
+    "v_cmp_ne_u32_e64 %[mb0], %[zero], %[b0]\n v_cmp_ne_u32_e64 %[mb1], %[zero], %[b1]\n"        \
+    "v_cmp_ne_u32_e64 %[mb2], %[zero], %[b2]\n v_cmp_ne_u32_e64 %[mb3], %[zero], %[b3]\n"
+#define PAM_BOTH_MASK_OPERANDS                                                                  \
+    [ma0] "=&s"(ma0), [ma1] "=&s"(ma1), [ma2] "=&s"(ma2), [ma3] "=&s"(ma3),                      \
+    [mb0] "=&s"(mb0), [mb1] "=&s"(mb1), [mb2] "=&s"(mb2), [mb3] "=&s"(mb3)
+__device__ __forceinline__ void pam_mac_4x4_skip_both(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr)
+{
+    uint32_t t0, t1, t2, t3;
+    uint64_t all, ma0, ma1, ma2, ma3, mb0, mb1, mb2, mb3;
     asm volatile(
-        "s_mov_b64 %[all], exec\n"
-        "v_cmp_ne_u32_e64 %[ma0], 0, %[a0]\n v_cmp_ne_u32_e64 %[ma1], 0, %[a1]\n"
-        "v_cmp_ne_u32_e64 %[ma2], 0, %[a2]\n v_cmp_ne_u32_e64 %[ma3], 0, %[a3]\n"
-        "v_cmp_ne_u32_e64 %[mb0], %[zero], %[b0]\n v_cmp_ne_u32_e64 %[mb1], %[zero], %[b1]\n"
-        "v_cmp_ne_u32_e64 %[mb2], %[zero], %[b2]\n v_cmp_ne_u32_e64 %[mb3], %[zero], %[b3]\n"
-        PAM_BOTH_ROW(0) PAM_BOTH_ROW(1) PAM_BOTH_ROW(2) PAM_BOTH_ROW(3)
+        "s_mov_b64 %[all], exec\n" PAM_BOTH_MASKS
+        PAM_BOTH_ROW(0, "all") PAM_BOTH_ROW(1, "all") PAM_BOTH_ROW(2, "all") PAM_BOTH_ROW(3, "all")
         "s_mov_b64 exec, %[all]\n"
-        : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]),
-          [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
-          [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]),
-          [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
-          [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [all] "=&s"(all),
-          [ma0] "=&s"(ma0), [ma1] "=&s"(ma1), [ma2] "=&s"(ma2), [ma3] "=&s"(ma3),
-          [mb0] "=&s"(mb0), [mb1] "=&s"(mb1), [mb2] "=&s"(mb2), [mb3] "=&s"(mb3), [pl] "+v"(pl), [pr] "+v"(pr)
-        : [a0] "v"(a.x), [a1] "v"(a.y), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w),
-          [zero] "s"(kZeroR));
-#undef PAM_BOTH_ROW
+        : PAM_ACC_OPERANDS, [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [all] "=&s"(all),
+          PAM_BOTH_MASK_OPERANDS, [pl] "+v"(pl), [pr] "+v"(pr)
+        : PAM_FRAGMENT_OPERANDS, [zero] "s"(kZeroR)
+        : "scc");
 }
+
+// ... and under a wavefront-uniform lane mask `run`, as pam_mac_4x4_under
+__device__ __forceinline__ void pam_mac_4x4_skip_both_under(float (&acc)[4][4], const u32x4& a, const u32x4& b, uint32_t& pl, uint32_t& pr,
+                                                            uint64_t run)
+{
+    uint32_t t0, t1, t2, t3;
+    uint64_t all, live, ma0, ma1, ma2, ma3, mb0, mb1, mb2, mb3;
+    asm volatile(
+        "s_mov_b64 %[all], exec\n s_and_b64 %[live], exec, %[run]\n" PAM_BOTH_MASKS
+        "s_and_b64 %[ma0], %[ma0], %[run]\n s_and_b64 %[ma1], %[ma1], %[run]\n"
+        "s_and_b64 %[ma2], %[ma2], %[run]\n s_and_b64 %[ma3], %[ma3], %[run]\n"
+        PAM_BOTH_ROW(0, "live") PAM_BOTH_ROW(1, "live") PAM_BOTH_ROW(2, "live") PAM_BOTH_ROW(3, "live")
+        "s_mov_b64 exec, %[all]\n"
+        : PAM_ACC_OPERANDS, [t0] "=&v"(t0), [t1] "=&v"(t1), [t2] "=&v"(t2), [t3] "=&v"(t3), [all] "=&s"(all), [live] "=&s"(live),
+          PAM_BOTH_MASK_OPERANDS, [pl] "+v"(pl), [pr] "+v"(pr)
+        : PAM_FRAGMENT_OPERANDS, [zero] "s"(kZeroR), [run] "s"(run)
+        : "scc");
+}
+#undef PAM_BOTH_ROW
+#undef PAM_BOTH_MASKS
+#undef PAM_BOTH_MASK_OPERANDS
 
 // The exact-backward products of a 4 x 4 micro-tile for one k (pam/cuda_kernels.cu:48-57): per product the slope
 // operand's bits plus the kept fraction, masked to sign and exponent, times the upstream gradient, added by one
 // fma.  DELTA_LEFT: the gradient is the left fragment (a) and the slope operand the right one (b); else the reverse.
 // Two statements of eight products; the LDS addresses pass through as in pam_mac_4x4.
-template <bool DELTA_LEFT>
+#define PAM_BWD_DL_LOW "v_add_u32 %[t0], %[b0], %[d00]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d01]\nv_fma_f32 %[c00], %[a0], %[t0], %[c00]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d02]\nv_fma_f32 %[c01], %[a0], %[t1], %[c01]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d03]\nv_fma_f32 %[c02], %[a0], %[t0], %[c02]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b0], %[d10]\nv_fma_f32 %[c03], %[a0], %[t1], %[c03]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d11]\nv_fma_f32 %[c10], %[a1], %[t0], %[c10]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d12]\nv_fma_f32 %[c11], %[a1], %[t1], %[c11]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d13]\nv_fma_f32 %[c12], %[a1], %[t0], %[c12]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c13], %[a1], %[t1], %[c13]\n"
+#define PAM_BWD_DL_HIGH "v_add_u32 %[t0], %[b0], %[d20]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d21]\nv_fma_f32 %[c20], %[a2], %[t0], %[c20]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d22]\nv_fma_f32 %[c21], %[a2], %[t1], %[c21]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d23]\nv_fma_f32 %[c22], %[a2], %[t0], %[c22]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b0], %[d30]\nv_fma_f32 %[c23], %[a2], %[t1], %[c23]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d31]\nv_fma_f32 %[c30], %[a3], %[t0], %[c30]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d32]\nv_fma_f32 %[c31], %[a3], %[t1], %[c31]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d33]\nv_fma_f32 %[c32], %[a3], %[t0], %[c32]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c33], %[a3], %[t1], %[c33]\n"
+#define PAM_BWD_DR_LOW "v_add_u32 %[t0], %[a0], %[d00]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a0], %[d01]\nv_fma_f32 %[c00], %[b0], %[t0], %[c00]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a0], %[d02]\nv_fma_f32 %[c01], %[b1], %[t1], %[c01]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a0], %[d03]\nv_fma_f32 %[c02], %[b2], %[t0], %[c02]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a1], %[d10]\nv_fma_f32 %[c03], %[b3], %[t1], %[c03]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a1], %[d11]\nv_fma_f32 %[c10], %[b0], %[t0], %[c10]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a1], %[d12]\nv_fma_f32 %[c11], %[b1], %[t1], %[c11]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a1], %[d13]\nv_fma_f32 %[c12], %[b2], %[t0], %[c12]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c13], %[b3], %[t1], %[c13]\n"
+#define PAM_BWD_DR_HIGH "v_add_u32 %[t0], %[a2], %[d20]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a2], %[d21]\nv_fma_f32 %[c20], %[b0], %[t0], %[c20]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a2], %[d22]\nv_fma_f32 %[c21], %[b1], %[t1], %[c21]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a2], %[d23]\nv_fma_f32 %[c22], %[b2], %[t0], %[c22]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a3], %[d30]\nv_fma_f32 %[c23], %[b3], %[t1], %[c23]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a3], %[d31]\nv_fma_f32 %[c30], %[b0], %[t0], %[c30]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a3], %[d32]\nv_fma_f32 %[c31], %[b1], %[t1], %[c31]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a3], %[d33]\nv_fma_f32 %[c32], %[b2], %[t0], %[c32]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c33], %[b3], %[t1], %[c33]\n"
+// UNDER: the statements run under the wavefront-uniform lane mask `run` (all ones or zero), as pam_mac_4x4_under.
+template <bool DELTA_LEFT, bool UNDER = false>
 __device__ __forceinline__ void pam_bwd_mac_4x4(float (&acc)[4][4], const uint32_t (&dfrac)[4][4], const u32x4& a, const u32x4& b,
-                                                uint32_t& pl, uint32_t& pr)
+                                                uint32_t& pl, uint32_t& pr, uint64_t run = 0)
 {
     uint32_t t0, t1;
+    uint64_t all;
     if (DELTA_LEFT) {
-    asm volatile("v_add_u32 %[t0], %[b0], %[d00]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d01]\nv_fma_f32 %[c00], %[a0], %[t0], %[c00]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d02]\nv_fma_f32 %[c01], %[a0], %[t1], %[c01]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d03]\nv_fma_f32 %[c02], %[a0], %[t0], %[c02]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b0], %[d10]\nv_fma_f32 %[c03], %[a0], %[t1], %[c03]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d11]\nv_fma_f32 %[c10], %[a1], %[t0], %[c10]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d12]\nv_fma_f32 %[c11], %[a1], %[t1], %[c11]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d13]\nv_fma_f32 %[c12], %[a1], %[t0], %[c12]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c13], %[a1], %[t1], %[c13]\n"
-                     : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
-                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl)
-                     : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]),
-                       [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
-        asm volatile("v_add_u32 %[t0], %[b0], %[d20]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d21]\nv_fma_f32 %[c20], %[a2], %[t0], %[c20]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d22]\nv_fma_f32 %[c21], %[a2], %[t1], %[c21]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d23]\nv_fma_f32 %[c22], %[a2], %[t0], %[c22]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b0], %[d30]\nv_fma_f32 %[c23], %[a2], %[t1], %[c23]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b1], %[d31]\nv_fma_f32 %[c30], %[a3], %[t0], %[c30]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[b2], %[d32]\nv_fma_f32 %[c31], %[a3], %[t1], %[c31]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[b3], %[d33]\nv_fma_f32 %[c32], %[a3], %[t0], %[c32]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c33], %[a3], %[t1], %[c33]\n"
-                     : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
-                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr)
-                     : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]),
-                       [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+        if constexpr (UNDER) {
+            asm volatile("s_mov_b64 %[all], exec\n s_and_b64 exec, exec, %[run]\n" PAM_BWD_DL_LOW "s_mov_b64 exec, %[all]\n"
+                         : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl), [all] "=&s"(all)
+                         : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]), [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w), [run] "s"(run)
+                         : "scc");
+            asm volatile("s_mov_b64 %[all], exec\n s_and_b64 exec, exec, %[run]\n" PAM_BWD_DL_HIGH "s_mov_b64 exec, %[all]\n"
+                         : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr), [all] "=&s"(all)
+                         : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w), [run] "s"(run)
+                         : "scc");
+        } else {
+            asm volatile(PAM_BWD_DL_LOW
+                         : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl)
+                         : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]), [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+            asm volatile(PAM_BWD_DL_HIGH
+                         : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr)
+                         : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+        }
     } else {
-    asm volatile("v_add_u32 %[t0], %[a0], %[d00]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a0], %[d01]\nv_fma_f32 %[c00], %[b0], %[t0], %[c00]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a0], %[d02]\nv_fma_f32 %[c01], %[b1], %[t1], %[c01]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a0], %[d03]\nv_fma_f32 %[c02], %[b2], %[t0], %[c02]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a1], %[d10]\nv_fma_f32 %[c03], %[b3], %[t1], %[c03]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a1], %[d11]\nv_fma_f32 %[c10], %[b0], %[t0], %[c10]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a1], %[d12]\nv_fma_f32 %[c11], %[b1], %[t1], %[c11]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a1], %[d13]\nv_fma_f32 %[c12], %[b2], %[t0], %[c12]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c13], %[b3], %[t1], %[c13]\n"
-                     : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]),
-                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl)
-                     : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]),
-                       [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
-        asm volatile("v_add_u32 %[t0], %[a2], %[d20]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a2], %[d21]\nv_fma_f32 %[c20], %[b0], %[t0], %[c20]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a2], %[d22]\nv_fma_f32 %[c21], %[b1], %[t1], %[c21]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a2], %[d23]\nv_fma_f32 %[c22], %[b2], %[t0], %[c22]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a3], %[d30]\nv_fma_f32 %[c23], %[b3], %[t1], %[c23]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a3], %[d31]\nv_fma_f32 %[c30], %[b0], %[t0], %[c30]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_add_u32 %[t0], %[a3], %[d32]\nv_fma_f32 %[c31], %[b1], %[t1], %[c31]\nv_and_b32 %[t0], 0xff800000, %[t0]\nv_add_u32 %[t1], %[a3], %[d33]\nv_fma_f32 %[c32], %[b2], %[t0], %[c32]\nv_and_b32 %[t1], 0xff800000, %[t1]\nv_fma_f32 %[c33], %[b3], %[t1], %[c33]\n"
-                     : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]),
-                       [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr)
-                     : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]),
-                       [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+        if constexpr (UNDER) {
+            asm volatile("s_mov_b64 %[all], exec\n s_and_b64 exec, exec, %[run]\n" PAM_BWD_DR_LOW "s_mov_b64 exec, %[all]\n"
+                         : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl), [all] "=&s"(all)
+                         : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]), [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w), [run] "s"(run)
+                         : "scc");
+            asm volatile("s_mov_b64 %[all], exec\n s_and_b64 exec, exec, %[run]\n" PAM_BWD_DR_HIGH "s_mov_b64 exec, %[all]\n"
+                         : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr), [all] "=&s"(all)
+                         : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w), [run] "s"(run)
+                         : "scc");
+        } else {
+            asm volatile(PAM_BWD_DR_LOW
+                         : [c00] "+v"(acc[0][0]), [c01] "+v"(acc[0][1]), [c02] "+v"(acc[0][2]), [c03] "+v"(acc[0][3]), [c10] "+v"(acc[1][0]), [c11] "+v"(acc[1][1]), [c12] "+v"(acc[1][2]), [c13] "+v"(acc[1][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pl)
+                         : [d00] "v"(dfrac[0][0]), [d01] "v"(dfrac[0][1]), [d02] "v"(dfrac[0][2]), [d03] "v"(dfrac[0][3]), [d10] "v"(dfrac[1][0]), [d11] "v"(dfrac[1][1]), [d12] "v"(dfrac[1][2]), [d13] "v"(dfrac[1][3]), [a0] "v"(a.x), [a1] "v"(a.y), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+            asm volatile(PAM_BWD_DR_HIGH
+                         : [c20] "+v"(acc[2][0]), [c21] "+v"(acc[2][1]), [c22] "+v"(acc[2][2]), [c23] "+v"(acc[2][3]), [c30] "+v"(acc[3][0]), [c31] "+v"(acc[3][1]), [c32] "+v"(acc[3][2]), [c33] "+v"(acc[3][3]), [t0] "=&v"(t0), [t1] "=&v"(t1), [p] "+v"(pr)
+                         : [d20] "v"(dfrac[2][0]), [d21] "v"(dfrac[2][1]), [d22] "v"(dfrac[2][2]), [d23] "v"(dfrac[2][3]), [d30] "v"(dfrac[3][0]), [d31] "v"(dfrac[3][1]), [d32] "v"(dfrac[3][2]), [d33] "v"(dfrac[3][3]), [a2] "v"(a.z), [a3] "v"(a.w), [b0] "v"(b.x), [b1] "v"(b.y), [b2] "v"(b.z), [b3] "v"(b.w));
+        }
     }
 }
+#undef PAM_BWD_DL_LOW
+#undef PAM_BWD_DL_HIGH
+#undef PAM_BWD_DR_LOW
+#undef PAM_BWD_DR_HIGH
 
 // Four work-groups per compute unit are what the LDS allows; the register budget follows (128 per lane), so that no
 // instance of the kernel falls to three wavefronts per SIMD.
@@ -576,7 +639,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             PlainStager<true> plus{(MODE == MODE_PAM ? 0u - kBias : 0u) + (shifted ? g.off_add : 0u)};
             if (kOffL && (MODE == MODE_PAM || shifted)) ll.store(lds_l[buf], tid, plus); else ll.store(lds_l[buf], tid, same);
             if (kOffR && (MODE == MODE_PAM || shifted)) rl.store(lds_r[buf], tid, plus); else rl.store(lds_r[buf], tid, same);
-            if (lane == 0) lds_flag[buf][wave] = 0u;
+            if (lane == 0) { lds_flag[buf][wave] = 0u; lds_odd_k[buf][wave] = 0u; }   // (the mask is read when another wavefront's verdict asks for it)
             return;
         }
         Stager<MODE, false> sl; Stager<MODE, true> sr;
@@ -710,9 +773,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_fmaf(u2f(a[i] + b[j]), keep[j], acc[i][j]);
     };
-    auto guarded_step = [&](int kk) __attribute__((always_inline)) {
-        uint32_t a[TM], b[TN];
-        fragment(kk, a, b);
+    // the products of one k-step by the full definition
+    auto guarded_products = [&](const uint32_t (&a)[TM], const uint32_t (&b)[TN]) __attribute__((always_inline)) {
         if (MODE == MODE_PAM) {
             Split sa[TM], sb[TN];
 #pragma unroll
@@ -732,6 +794,11 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                 if (MODE == MODE_BWD_DL) acc[i][j] += bwd_product_general(dfrac[i][j], b[j], u2f(a[i]));
                 else if (MODE == MODE_BWD_DR) acc[i][j] += bwd_product_general(dfrac[i][j], a[i], u2f(b[j]));
             }
+    };
+    auto guarded_step = [&](int kk) __attribute__((always_inline)) {
+        uint32_t a[TM], b[TN];
+        fragment(kk, a, b);
+        guarded_products(a, b);
     };
 
     // a full k-tile of in-range values: fragments for step kk+1 are read from LDS while step kk is computed
@@ -804,6 +871,44 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     };
     constexpr bool kSkips = MODE == MODE_PAM && TM == 4 && TN == 4;
 
+    // a full k-tile some of whose k-steps hold a value in need of the full definition (bit k of `odd`): a rolled loop
+    // over the k-steps in which every step passes through the plain block (the skipping one if the tile holds zeros
+    // too, ZEROS) -- under an empty lane mask in the marked steps, whose products the full definition then adds.
+    auto mixed_tile = [&](uint32_t odd, auto holds_zeros) __attribute__((always_inline)) {
+        if constexpr (MODE != MODE_STD && TM == 4 && TN == 4) {
+            constexpr bool ZEROS = decltype(holds_zeros)::value;
+            typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
+            uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+#pragma unroll 1
+            for (int kk = 0; kk < BK; ++kk) {
+                const u32x4 va = *reinterpret_cast<LdsVec>(pl), vb = *reinterpret_cast<LdsVec>(pr);
+                pl += LDL * 4; pr += LDR * 4;
+                // a marked step concerns the wavefronts whose lanes hold one of its odd values: 16 of a work-group's 256
+                // lanes for a value of the left operand, 16 per wavefront for one of the right operand
+                bool marked = ((odd >> kk) & 1u) != 0;
+                if (__builtin_expect(marked, 0)) {
+                    constexpr uint32_t kUnstage = MODE == MODE_PAM ? kBias : 0u;      // the right operand is staged less the bias
+                    auto is_odd = [](uint32_t u) { return (u & ~kSign) != 0 && ((u >> 23) & 0xffu) - 64u > 126u; };
+                    const bool mine = is_odd(va.x) || is_odd(va.y) || is_odd(va.z) || is_odd(va.w) || is_odd(vb.x + kUnstage)
+                                   || is_odd(vb.y + kUnstage) || is_odd(vb.z + kUnstage) || is_odd(vb.w + kUnstage);
+                    marked = __ballot(mine) != 0ull;
+                }
+                const uint32_t half = __builtin_amdgcn_readfirstlane(marked ? 0u : ~0u);     // (keeps the mask in scalar registers)
+                const uint64_t run = ((uint64_t)half << 32) | half;
+                if constexpr (MODE == MODE_PAM) {
+                    if constexpr (ZEROS) pam_mac_4x4_skip_both_under(acc, va, vb, pl, pr, run);
+                    else pam_mac_4x4_under(acc, va, vb, pl, pr, run);
+                } else {
+                    pam_bwd_mac_4x4<MODE == MODE_BWD_DL, true>(acc, dfrac, va, vb, pl, pr, run);
+                }
+                if (__builtin_expect(marked, 0)) {
+                    const uint32_t a[4] = {va.x, va.y, va.z, va.w}, b[4] = {vb.x, vb.y, vb.z, vb.w};
+                    guarded_products(a, b);
+                }
+            }
+        }
+    };
+
     int t = 0;
     while (t < ktiles) {
         begin_tile(t);
@@ -845,6 +950,12 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             for (int w = 0; w < NW; ++w) odd |= lds_odd_k[t & 1][w];
             odd = __builtin_amdgcn_readfirstlane(odd);
             const bool zeros = MODE == MODE_PAM && (verdict & (kZerosL | kZerosR)) != 0;    // somewhere in the tile
+            if (MODE != MODE_STD && TM == 4 && TN == 4 && kcount == BK) {
+                if (zeros) mixed_tile(odd, std::true_type()); else mixed_tile(odd, std::false_type());
+                end_tile(t);
+                ++t;
+                continue;
+            }
 #pragma unroll 1
             for (int kk = 0; kk < kcount; ++kk) {
                 if ((odd >> kk) & 1u) guarded_step(kk);
