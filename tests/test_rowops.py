@@ -307,7 +307,7 @@ def test_gpu_softmax_special_values(oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n", [100, 700, 2000, 20000])
+@pytest.mark.parametrize("n", [100, 150, 350, 700, 2000, 20000])
 def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n):
     """All-exact gradients without an offset first run on unchecked arithmetic: inputs and upstream gradients at and
     beyond the edges of what that accepts (zeros, subnormals, huge and tiny values, inf, NaN, a variance of exactly 1)."""
