@@ -639,7 +639,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             PlainStager<true> plus{(MODE == MODE_PAM ? 0u - kBias : 0u) + (shifted ? g.off_add : 0u)};
             if (kOffL && (MODE == MODE_PAM || shifted)) ll.store(lds_l[buf], tid, plus); else ll.store(lds_l[buf], tid, same);
             if (kOffR && (MODE == MODE_PAM || shifted)) rl.store(lds_r[buf], tid, plus); else rl.store(lds_r[buf], tid, same);
-            if (lane == 0) { lds_flag[buf][wave] = 0u; lds_odd_k[buf][wave] = 0u; }   // (the mask is read when another wavefront's verdict asks for it)
+            if (lane == 0) lds_flag[buf][wave] = 0u;      // (its k mask keeps an older value: readers go by the flag)
             return;
         }
         Stager<MODE, false> sl; Stager<MODE, true> sr;
@@ -947,7 +947,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             // some value of the k-tile needs the full definition: only the k-steps that hold one pay for it
             uint32_t odd = 0u;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) odd |= lds_odd_k[t & 1][w];
+            for (int w = 0; w < NW; ++w) odd |= lds_flag[t & 1][w] >= kGuarded ? lds_odd_k[t & 1][w] : 0u;     // only those wavefronts wrote one
             odd = __builtin_amdgcn_readfirstlane(odd);
             const bool zeros = MODE == MODE_PAM && (verdict & (kZerosL | kZerosR)) != 0;    // somewhere in the tile
             if (MODE != MODE_STD && TM == 4 && TN == 4 && kcount == BK) {
