@@ -139,3 +139,13 @@ class Linear(torch.nn.Linear):
             parts.append(f"offset={self.offset:0.5f}")
         parts.append(f"approx_bwd={self.approx_bwd}")
         return ", ".join(parts)
+
+
+def __getattr__(name):
+    # The reference keeps conv2d, conv2d_group, Conv2d, mean, softmax, logsumexp, log_softmax, layer_norm and LayerNorm in
+    # this module too (pam/pam_ops.py:118-404); here they live in `composites`, which imports this module, so they are
+    # looked up on first use: `pam.pam_ops.softmax` and `from pam.pam_ops import LayerNorm` work as they do there.
+    from . import composites
+    if name in composites.__all__:
+        return getattr(composites, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

@@ -3,6 +3,8 @@ shared/modules/factories.py:128-265 and pam/__init__.py:8-10 read must resolve f
 op tables must be bound to the same objects."""
 import inspect
 
+import pytest
+
 import torch
 
 import pam
@@ -47,3 +49,17 @@ def test_function_dict_binds_to_the_package():
     # the dict form filters keywords the op does not take (fairseq passes dtype= to softmax)
     custom = factories.get_function_dict({"type": "pam", "dkwargs": {"approx_bwd": True}, "okwargs": {}})
     assert set(custom) == set(table)
+
+
+def test_pam_ops_module_serves_every_name_of_the_reference_module():
+    """pam/pam_ops.py defines the primitives and the compositions in one module (its def / class names, :16-404)."""
+    import importlib
+    ops = importlib.import_module("pam.pam_ops")
+    for name in ("mul", "div", "exp", "exp2", "log", "log2", "pow", "matmul", "bmm", "linear", "conv2d", "conv2d_group",
+                 "Conv2d", "Linear", "mean", "softmax", "logsumexp", "log_softmax", "layer_norm", "LayerNorm"):
+        assert callable(getattr(ops, name)), name
+    from pam.pam_ops import softmax, LayerNorm          # noqa: F401
+    import pam
+    assert ops.softmax is pam.softmax and ops.Conv2d is pam.Conv2d
+    with pytest.raises(AttributeError):
+        ops.no_such_name
