@@ -543,7 +543,8 @@ void pamo_logsumexp_fwd(const float *x, float *lse, float *y, long rows, long n,
         for (long i = 0; i < n; ++i) { volatile float t = scaled_x(x[r * n + i], off, 0) - shift; e[i] = exp2_op(t, off); }
         float total = row_sum_fixed(e, n);
         free(e);
-        volatile float s = shift + log2_op(total, off);
+        /* log2 of the total is called without the keyword arguments (pam/pam_ops.py:341): no offset */
+        volatile float s = shift + log2_op(total, 1.0f);
         float out = pad_off(s, LOG2_E, off);
         if (lse) lse[r] = out;
         if (y) for (long i = 0; i < n; ++i) { volatile float d = x[r * n + i] - out; y[r * n + i] = d; }
@@ -610,9 +611,11 @@ void pamo_logsumexp_bwd(const float *x, const float *grad, float shift, float *d
         float total = row_sum_fixed(e, n);
         float g_out;
         if (log_softmax) { volatile float s = row_sum_fixed(grad + r * n, n); g_out = -s; } else g_out = grad[r];
-        volatile float u = shift + log2_op(total, off);
+        /* log2(total) carries no keyword arguments in the reference (pam/pam_ops.py:341): no offset, and the exact
+         * gradient (pa_log_bwd) whatever approx_bwd says */
+        volatile float u = shift + log2_op(total, 1.0f);
         float du = g_div_da(k, u, LOG2_E, g_out);
-        float dtotal = g_log2_dx(k, total, du);
+        float dtotal = palog_bwd(total, du, 1.0f, 1.0f);
         for (long i = 0; i < n; ++i) {
             volatile float t = scaled_x(xr[i], off, 0) - shift;
             float d = g_mul_da(k, xr[i], LOG2_E, g_exp2_dx(k, t, dtotal));

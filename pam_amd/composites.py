@@ -80,7 +80,9 @@ def logsumexp(x, dim, keepdim=False, *, offset=None, approx_bwd=False, use_kerne
         return fused.logsumexp(x, keepdim, offset, approx_bwd)
     weights, shift = _scaled_exp2(x, kw, None)
     total = torch.sum(weights, dim=dim, keepdim=keepdim)
-    return div(shift + log2(total, **kw), _LOG2_E, **kw)
+    # the reference takes log2 of the total without its keyword arguments (pam/pam_ops.py:341): no offset there, and
+    # that log2's gradient is the exact one whatever approx_bwd says
+    return div(shift + log2(total), _LOG2_E, **kw)
 
 
 def log_softmax(x, dim=None, *, offset=None, approx_bwd=False, use_kernel=True):

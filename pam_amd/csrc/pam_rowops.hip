@@ -229,6 +229,8 @@ struct Checked {
     __device__ __forceinline__ float div(float a, float b) { return pad_div_off(a, b, o.off, o.has); }
     __device__ __forceinline__ float exp2(float t) { return exp2_entry(t, o.off, o.has); }
     __device__ __forceinline__ float log2(float v) { return log2_entry(v, o.off, o.has); }
+    // log2 as logsumexp calls it: without the keyword arguments, hence never with the offset (pam/pam_ops.py:341)
+    __device__ __forceinline__ float log2_plain(float v) { return log2_entry(v, 1.0f, false); }
     __device__ __forceinline__ float root(float v) { return pow_half(v, o.off, o.has); }
     // 0 (/) b for an element whose weight is exactly zero
     __device__ __forceinline__ float zero_over(float b) { return pad_div_off(0.0f, b, o.off, o.has); }
@@ -246,6 +248,7 @@ struct Unchecked {
     __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, o.has, sp); }
     __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, o.has, sp); }
     __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float log2_plain(float v) { return log2_entry_unchecked(v, 1.0f, false, sp); }
     __device__ __forceinline__ float root(float v) { return pow_half_unchecked(v, o.off, o.has, sp); }
     __device__ __forceinline__ float zero_over(float) { return 0.0f; }      // the divisor is a positive normal number when valid
     __device__ __forceinline__ bool valid() const { return sp.normal(); }
@@ -624,7 +627,7 @@ __device__ __forceinline__ float logsumexp_row(const float (&xv)[CH], float shif
         const float e = m.exp2(inside ? t : 0.5f);
         if (inside) p = p + e;
     }
-    return m.div(shift + m.log2(lay.sum(p)), kLog2E);
+    return m.div(shift + m.log2_plain(lay.sum(p)), kLog2E);
 }
 
 template <int CH>
@@ -660,7 +663,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                     const float e = m.exp2(inside ? m.mul_const(v, kLog2E) - shift : 0.5f);
                     if (inside) p = p + e;
                 });
-                return m.div(shift + m.log2(wave_sum(p)), kLog2E);
+                return m.div(shift + m.log2_plain(wave_sum(p)), kLog2E);
             };
             Unchecked u{o, Span()};
             float out = sweep(u);
@@ -788,8 +791,19 @@ struct GradChecked {
     { return ap.e ? mul(mul(exp2(x), kLn2), g) : exp2_entry_bwd(x, g, o.off, o.has); }
     __device__ __forceinline__ float log2_dx(float x, float g)
     { return ap.e ? div(div(g, x), kLn2) : log2_entry_bwd(x, g, o.off, o.has); }
+    // logsumexp's log2 of the row total: called without the keyword arguments (pam/pam_ops.py:341), so it takes no
+    // offset and its gradient is the exact one whatever approx_bwd says
+    __device__ __forceinline__ float log2_plain(float v) { return log2_entry(v, 1.0f, false); }
+    __device__ __forceinline__ float log2_plain_dx(float x, float g) { return log2_entry_bwd(x, g, 1.0f, false); }
     __device__ __forceinline__ bool valid() const { return true; }
 };
+// the exact gradient of log2 without an offset in the normal range: 2^-e(x) g (pam/cuda_kernels.cu:132-136)
+__device__ __forceinline__ float log2_exact_dx_unchecked(float x, float g, Span& sp)
+{
+    const uint32_t xi = f2u(x);                                            // positive (a sign bit reads as too large), below 2^127
+    sp.see(xi); sp.see(xi + 0x00800000u);
+    return u2f((254u << 23) - (xi & kExpo)) * g;
+}
 struct GradUnchecked {
     Offset o; Span sp;
     __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, o.has, sp); }
@@ -802,6 +816,8 @@ struct GradUnchecked {
     __device__ __forceinline__ float div_db(float a, float b, float g) { return -mul(div(div(a, b), b), g); }
     __device__ __forceinline__ float exp2_dx(float x, float g) { return mul(mul(exp2(x), kLn2), g); }
     __device__ __forceinline__ float log2_dx(float x, float g) { return div(div(g, x), kLn2); }
+    __device__ __forceinline__ float log2_plain(float v) { return log2_entry_unchecked(v, 1.0f, false, sp); }
+    __device__ __forceinline__ float log2_plain_dx(float x, float g) { return log2_exact_dx_unchecked(x, g, sp); }
     __device__ __forceinline__ bool valid() const { return sp.normal(); }
 };
 
@@ -833,12 +849,9 @@ struct GradUncheckedExact {
         return -u2f(ratio | (oi & kSign)) * g;
     }
     __device__ __forceinline__ float exp2_dx(float x, float g) { return u2f(f2u(exp2(x)) & ~kMant) * g; }
-    __device__ __forceinline__ float log2_dx(float x, float g)
-    {
-        const uint32_t xi = f2u(x);                                            // positive (a sign bit reads as too large), below 2^127
-        sp.see(xi); sp.see(xi + 0x00800000u);
-        return u2f((254u << 23) - (xi & kExpo)) * g;
-    }
+    __device__ __forceinline__ float log2_dx(float x, float g) { return log2_exact_dx_unchecked(x, g, sp); }
+    __device__ __forceinline__ float log2_plain(float v) { return log2(v); }
+    __device__ __forceinline__ float log2_plain_dx(float x, float g) { return log2_dx(x, g); }
     __device__ __forceinline__ bool valid() const { return sp.normal(); }
 };
 
@@ -860,9 +873,9 @@ __device__ __forceinline__ void logsumexp_grad_row(const float (&xv)[CH], const 
     }
     const float total = lay.sum(p);
     const float g_out = log_softmax ? -lay.sum(q) : g_row;         // log_softmax is the same for every thread of a launch         // x - lse: the broadcast lse collects -sum(gy)
-    const float u = shift + m.log2(total);
+    const float u = shift + m.log2_plain(total);
     const float du = m.div_da(u, kLog2E, g_out);
-    const float dtotal = m.log2_dx(total, du);
+    const float dtotal = m.log2_plain_dx(total, du);
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const bool inside = lay.index(c) < n;
@@ -928,9 +941,9 @@ __device__ __forceinline__ void logsumexp_grad_stream(const float* __restrict__ 
     }
     const float total = wave_sum(p);
     const float g_out = log_softmax ? -wave_sum(q) : g_row;
-    const float u = shift + m.log2(total);
+    const float u = shift + m.log2_plain(total);
     const float du = m.div_da(u, kLog2E, g_out);
-    const float dtotal = m.log2_dx(total, du);
+    const float dtotal = m.log2_plain_dx(total, du);
     for (int base = 0; base < n; base += 64 * U) {
         float xv[U], gy[U];
 #pragma unroll

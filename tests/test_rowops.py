@@ -100,11 +100,34 @@ def softmax_grad_chain(o, x, g, off, approx):
 
 
 def logsumexp_chain(o, x, off):
+    """pam/pam_ops.py:333-342: the offset goes to mul, exp2 and div; log2 of the row total is called bare."""
     s = o.pam(x, C, off)
     shift = np.floor(s.max())
     e = o.pa_exp((s - shift).astype(np.float32), 2.0, off)
     total = fixed_sum(e)
-    return o.pad((shift + o.pa_log(total, 2.0, off)).astype(np.float32), C, off)
+    return o.pad((shift + o.pa_log(total, 2.0, None)).astype(np.float32), C, off)
+
+
+def logsumexp_grad_chain(o, x, g_out, off, approx):
+    """Autograd's walk back through pam/pam_ops.py:333-342 with the backward formula of each Function
+    (pam/cuda_bindings.py:43-57, 78-97, 224-239, 262-276): div -> add -> log2 -> sum -> exp2 -> subtract -> mul.
+    log2 was called without keyword arguments, so its gradient is pa_log_bwd without an offset, always."""
+    approx_a, _, approx_e = approx
+    s = o.pam(x, C, off)
+    shift = np.floor(s.max())
+    t = (s - shift).astype(np.float32)
+    e = o.pa_exp(t, 2.0, off)
+    total = fixed_sum(e)
+    u = (shift + o.pa_log(total, 2.0, None)).astype(np.float32)
+    inv = o.pad(np.ones_like(u), np.full_like(u, C), off)
+    d_u = o.pam(inv, g_out, off) if approx_a else o.pam_bwd(u, inv, g_out, None)
+    d_total = o.pa_log_bwd(total, d_u, 2.0, None)
+    d_e = np.broadcast_to(d_total[:, None], x.shape).astype(np.float32)
+    if approx_e:
+        d_t = o.pam(o.pam(o.pa_exp(t, 2.0, off), LN2, off), d_e, off)
+    else:
+        d_t = o.pa_exp_bwd(t, d_e, 2.0, off)
+    return o.pam(d_t, C, off) if approx_a else o.pam_bwd(x, np.full_like(x, C), d_t, off)
 
 
 def layer_norm_chain(o, x, w, b, eps, off):
@@ -243,6 +266,66 @@ def test_logsumexp_and_layer_norm_gradient_chains_are_what_autograd_does(on_cpu,
             if ww is not None:
                 close(terms.sum(0), wt.grad.numpy())
                 close(g_full.sum(0), bt.grad.numpy())
+
+
+def reference_text_logsumexp(x, dim, keepdim=False, **pam_kwargs):
+    """The reference's logsumexp as its source reads (pam/pam_ops.py:333-342), on the op library's primitives: the
+    keyword arguments (offset, approx_bwd) go to the product, to exp2 and to the quotient -- the log2 of the summed
+    weights gets none of them (:341).  Independent of `composites.logsumexp` on purpose."""
+    k = math.log2(math.e)
+    scaled = pam_ops.mul(x, k, **pam_kwargs)
+    with torch.no_grad():
+        shift = torch.floor(torch.max(scaled))
+    weights = pam_ops.exp2(scaled - shift, **pam_kwargs)
+    total = torch.sum(weights, dim=dim, keepdim=keepdim)
+    bare_log2 = pam_ops.log2(total)                       # no offset, exact gradient
+    return pam_ops.div(shift + bare_log2, k, **pam_kwargs)
+
+
+@pytest.mark.parametrize("approx", [False, True, (True, False), (False, True)])
+@pytest.mark.parametrize("off", [None, OFF])
+def test_logsumexp_is_the_chain_the_reference_text_writes(on_cpu, off, approx):
+    """Values and gradients of logsumexp / log_softmax in three restatements -- the unfused composition of this
+    package, the oracle's fused restatement (what the HIP row kernels are compared with) and the primitives' backward
+    formulas chained by hand -- against the chain as the reference's source text has it.  A restatement that hands the
+    offset or approx_bwd to the inner log2 differs by percents (forward with an offset, gradient with approx_bwd) and fails."""
+    o = on_cpu
+    x = rows_case(31, 6, 40, masks=False)
+    rng = np.random.RandomState(32)
+    g_rows = rng.standard_normal(6).astype(np.float32); g_full = rng.standard_normal(x.shape).astype(np.float32)
+
+    def close(got, want, what, tol=1e-5):
+        scale = np.abs(want).max()
+        assert np.isfinite(want).all() and np.abs(got - want).max() <= tol * scale, (what, np.abs(got - want).max(), scale)
+
+    xt = torch.from_numpy(x.copy()).requires_grad_()
+    ref = reference_text_logsumexp(xt, -1, offset=off, approx_bwd=approx)
+    ref.backward(torch.from_numpy(g_rows))
+    ref_val, ref_grad = ref.detach().numpy(), xt.grad.numpy().copy()
+    xt = torch.from_numpy(x.copy()).requires_grad_()
+    (xt - reference_text_logsumexp(xt, -1, keepdim=True, offset=off, approx_bwd=approx)).backward(torch.from_numpy(g_full))
+    ref_ls_grad = xt.grad.numpy().copy()
+    shift = np.floor(o.pam(x, C, off).max())
+
+    # this package's unfused composition: the same torch ops, so the same bits
+    xt = torch.from_numpy(x.copy()).requires_grad_()
+    y = composites.logsumexp(xt, dim=-1, offset=off, approx_bwd=approx)
+    y.backward(torch.from_numpy(g_rows))
+    assert_same_bits(y.detach().numpy(), ref_val, "composites.logsumexp")
+    assert_same_bits(xt.grad.numpy(), ref_grad, "composites.logsumexp gradient")
+    xt = torch.from_numpy(x.copy()).requires_grad_()
+    composites.log_softmax(xt, dim=-1, offset=off, approx_bwd=approx).backward(torch.from_numpy(g_full))
+    assert_same_bits(xt.grad.numpy(), ref_ls_grad, "composites.log_softmax gradient")
+
+    # the oracle's fused restatement and the hand-chained formulas: fixed-order row sums instead of torch's
+    lse, ls = o.logsumexp_fwd(x, off, with_log_softmax=True)
+    close(lse, ref_val, "oracle logsumexp", 2e-6)
+    close(ls, x - ref_val[:, None], "oracle log_softmax", 2e-6)
+    assert_same_bits(lse, logsumexp_chain(o, x, off), "oracle logsumexp vs hand chain")
+    close(o.logsumexp_bwd(x, g_rows, shift, off, _flags(approx)), ref_grad, "oracle logsumexp gradient")
+    close(o.logsumexp_bwd(x, g_full, shift, off, _flags(approx), log_softmax=True), ref_ls_grad, "oracle log_softmax gradient")
+    assert_same_bits(o.logsumexp_bwd(x, g_rows, shift, off, _flags(approx)), logsumexp_grad_chain(o, x, g_rows, off, _flags(approx)),
+                     "oracle logsumexp gradient vs hand chain")
 
 
 # ------------------------------------------------------------------ GPU: HIP kernels == oracle fused
