@@ -358,10 +358,6 @@ __global__ __launch_bounds__(kThreads) void adam_scalar_kernel(float* __restrict
 extern "C" {
 
 int pam_hip_abi_version(void) { return PAM_HIP_ABI_VERSION; }
-#ifndef PAM_HIP_SOURCE_HASH
-#define PAM_HIP_SOURCE_HASH "unstamped"
-#endif
-const char* pam_hip_source_hash(void) { return PAM_HIP_SOURCE_HASH; }
 const char* pam_hip_last_error(void) { return pamhost::error_buffer(); }
 
 int pam_hip_device_info(int* compute_units, int* clock_khz)
