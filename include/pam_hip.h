@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define PAM_HIP_ABI_VERSION 1
+#define PAM_HIP_ABI_VERSION 2
 
 enum {
     PAM_HIP_OK = 0,
@@ -92,26 +92,28 @@ int pam_hip_pa_log_bwd(const float *x, const float *dy, float *dx, size_t n, flo
 #define PAM_HIP_MAT(name) const float *name, long name##_sb, long name##_sr, long name##_sc
 #define PAM_HIP_OUT(name) float *name, long name##_sb, long name##_sr, long name##_sc
 
-/* Scratch needed by the split-K path that large-K, small-output products use (0 if the
- * shape does not use it).  Passing workspace == NULL to the calls below is always valid
- * and simply disables that path. */
+/* Scratch for a product of this shape: the words of the queues that the work-groups of a launch draw their output
+ * tiles from and, for shapes with few output tiles and long k (their tiles' k ranges are cut into pieces that
+ * different work-groups sum), the pieces and one arrival word per tile.  16-byte aligned.  A workspace needs no
+ * preparation before its first use (any contents), every call leaves it ready for the next one, and two products
+ * that overlap in time must not share one.  Passing workspace == NULL (or fewer bytes) to the calls below is
+ * always valid: tiles are then never cut and every work-group computes one tile, at some cost in speed. */
 size_t pam_hip_gemm_workspace_bytes(long batch, long m, long n, long k);
 
 /* The accumulation order a product of this shape uses when the workspace is supplied.
  * k is cut into chunks of *k_chunk consecutive values (a multiple of 16; the last chunk may
  * be shorter).  Each chunk is summed in ascending k from +0 into one fp32 accumulator per
- * output.  Every *k_group consecutive chunk sums are added in ascending order, and those
- * group sums are added in ascending order from +0.  One chunk (k_chunk >= k) is the order
- * of the reference kernel (pam/cuda_kernels.cu:601, 608-627).  Without a workspace the
- * order is a single group of *k_group chunks of ceil(ceil(k/16) / k_group) * 16. */
-int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_chunk, int *k_group);
+ * output, and the chunk sums are added in ascending order from +0.  One chunk (k_chunk >= k) is the
+ * order of the reference kernel (pam/cuda_kernels.cu:601, 608-627), which is also the order without a
+ * workspace. */
+int pam_hip_gemm_plan(long batch, long m, long n, long k, int *k_chunk);
 
 /* Y[m,n] = sum_k A[m,k] (*) B[k,n]            replaces pam_matmul_fwd (matmul_caller<&pam,false>, :703-718) */
 int pam_hip_pam_matmul_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
                            float *y, long y_sr, long y_sc, long m, long n, long k, float offset,
                            void *workspace, size_t workspace_bytes, void *stream);
 /* The same product for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The split-k partial tiles go to an
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  What a workspace would hold goes to an
  * array of PAM_HIP_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, for the life of
  * the process; the call allocates and frees nothing.  Results are bit-identical to pam_hip_pam_matmul_fwd with
  * a workspace of pam_hip_gemm_workspace_bytes(1, m, n, k).  A shape that needs more scratch than the array is
@@ -122,7 +124,7 @@ int pam_hip_pam_matmul_fwd_noalloc(const float *a, long a_sr, long a_sc, const f
                                    float *y, long y_sr, long y_sc, long m, long n, long k, float offset, void *stream);
 /* Y = A (x) B + bias[column]: the product followed by the bias add of pam.linear
  * (pam/pam_ops.py:107-115) in one pass; the bias is added once to the finished sum (after the chunk
- * sums when k is split), which is what the separate add computes.  bias NULL = no bias. */
+ * sums when k is cut), which is what the separate add computes.  bias NULL = no bias. */
 int pam_hip_pam_linear_fwd(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc, const float *bias,
                            float *y, long y_sr, long y_sc, long m, long n, long k, float offset,
                            void *workspace, size_t workspace_bytes, void *stream);

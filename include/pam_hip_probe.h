@@ -19,9 +19,10 @@ int pam_hip_issue_probe(const void *seed, float *out, int blocks, int iters, voi
  * tm x tn micro-tile (4x4, 8x4, 8x8); each lane iters * 32 * tm * tn pairs. */
 int pam_hip_issue_probe_lds(const void *seed, float *out, int blocks, int iters, int tm, int tn, void *stream);
 
-/* Tuning hook for experiments: forces the k-tile depth (16 or 32; 0 = automatic) and the number of
- * k chunks (0 = automatic) of the matrix products for the calling thread; pam_hip_gemm_plan and pam_hip_gemm_workspace_bytes follow the forced values. */
-void pam_hip_set_tuning(int k_tile, int k_chunks);
+/* Tuning hook for experiments: forces the k-tile depth (16 or 32; 0 = automatic) and the number of pieces every
+ * output tile's k range is cut into (0 = automatic; 1 = whole tiles) of the matrix products for the calling thread;
+ * pam_hip_gemm_plan and pam_hip_gemm_workspace_bytes follow the forced values. */
+void pam_hip_set_tuning(int k_tile, int pieces);
 
 #ifdef __cplusplus
 }

@@ -44,7 +44,7 @@ _SIGNATURES = {
     "pam_hip_pa_log_fwd": ([_p, _p, _z, _f, _f, _p], _i),
     "pam_hip_pa_log_bwd": ([_p, _p, _p, _z, _f, _f, _p], _i),
     "pam_hip_gemm_workspace_bytes": ([_l, _l, _l, _l], _z),
-    "pam_hip_gemm_plan": ([_l, _l, _l, _l, ctypes.POINTER(_i), ctypes.POINTER(_i)], _i),
+    "pam_hip_gemm_plan": ([_l, _l, _l, _l, ctypes.POINTER(_i)], _i),
     "pam_hip_pam_matmul_fwd": (_MAT2 * 3 + [_l, _l, _l, _f, _p, _z, _p], _i),
     "pam_hip_pam_matmul_fwd_noalloc": (_MAT2 * 3 + [_l, _l, _l, _f, _p], _i),
     "pam_hip_pam_linear_fwd": (_MAT2 * 2 + [_p] + _MAT2 + [_l, _l, _l, _f, _p, _z, _p], _i),
@@ -88,7 +88,7 @@ def load_library():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = restype
-        if lib.pam_hip_abi_version() != 1:
+        if lib.pam_hip_abi_version() != 2:
             raise RuntimeError("libpam_hip.so has an unexpected ABI version")
         _lib = lib
     return _lib
@@ -113,13 +113,27 @@ def device_info():
 
 
 def gemm_plan(batch, m, n, k):
-    """(k_chunk, k_group): the fixed accumulation order used for this shape (see include/pam_hip.h)."""
-    c, g = _i(0), _i(0)
-    _call("pam_hip_gemm_plan", batch, m, n, k, ctypes.byref(c), ctypes.byref(g))
-    return c.value, g.value
+    """k_chunk: the fixed accumulation order used for this shape (see pam_hip_gemm_plan in include/pam_hip.h)."""
+    c = _i(0)
+    _call("pam_hip_gemm_plan", batch, m, n, k, ctypes.byref(c))
+    return c.value
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+# The matrix products' scratch (queue words, pieces of cut tiles): one buffer per device and stream, kept and grown
+# as needed -- products on one stream run one after the other and each leaves the buffer ready for the next, and the
+# buffer is never handed to anything else, so its words are always either fresh zeros or what a product left.
+_workspaces = {}
+
+
+def _gemm_workspace(device, nbytes):
+    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() * 4 < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20) // 4 + 64, dtype=torch.float32, device=device)
+        _workspaces[key] = ws
+    return ws
 
 
 def _stream():
@@ -293,7 +307,7 @@ class HipKernels:
         with _on(L.device):
             lib = load_library()
             ws_bytes = lib.pam_hip_gemm_workspace_bytes(batch, m, n, k)
-            ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=L.device) if ws_bytes else None
+            ws = _gemm_workspace(L.device, ws_bytes) if ws_bytes else None
             args = []
             for t in ops:
                 args += cls._mat(t, batched)

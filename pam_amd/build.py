@@ -15,7 +15,9 @@ import tempfile
 
 HERE = pathlib.Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
-SOURCES = [CSRC / "pam_gemm.hip", CSRC / "pam_rowops.hip", CSRC / "pam_elementwise.hip", CSRC / "pam_probe.hip"]   # slowest first
+SOURCES = sorted(CSRC.glob("pam_gemm_inst_*.hip")) + [CSRC / "pam_rowops.hip", CSRC / "pam_gemm.hip", CSRC / "pam_elementwise.hip",
+                                                      CSRC / "pam_probe.hip"]   # slowest first
+JOBS = 8
 STAMP_SOURCE = CSRC / "pam_stamp.cpp"
 LIB = HERE / "lib" / "libpam_hip.so"
 
@@ -36,6 +38,18 @@ def _run(cmd, verbose):
         raise RuntimeError("hipcc failed:\n" + err)
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def _with_includes(src, seen=None):
+    """src and the project headers it includes ("..." includes, followed recursively), in a fixed order."""
+    seen = [] if seen is None else seen
+    src = src.resolve()
+    if src in seen or not src.is_file():
+        return seen
+    seen.append(src)
+    for name in re.findall(r'^\s*#\s*include\s+"([^"]+)"', src.read_text(), flags=re.M):
+        _with_includes(src.parent / name, seen)
+    return seen
 
 
 def source_files():
@@ -85,17 +99,16 @@ def build(verbose=False, object_dir=None):
     the default compiles everything)."""
     LIB.parent.mkdir(exist_ok=True)
     stamp = f'-DPAM_HIP_SOURCE_HASH="{source_hash()}"'
-    headers = b"".join(f.read_bytes() for f in source_files() if f.suffix == ".h")
     with tempfile.TemporaryDirectory() as tmp:
         out = pathlib.Path(object_dir) if object_dir else pathlib.Path(tmp)
         out.mkdir(parents=True, exist_ok=True)
         jobs, objects = [], []
-        with concurrent.futures.ThreadPoolExecutor(len(SOURCES) + 1) as pool:
+        with concurrent.futures.ThreadPoolExecutor(JOBS) as pool:
             for src in SOURCES + [STAMP_SOURCE]:
                 obj = out / (src.stem + ".o")
                 objects.append(str(obj))
                 flags = FLAGS + ([stamp] if src == STAMP_SOURCE else [])
-                key = hashlib.sha256(" ".join(flags).encode() + src.read_bytes() + headers).hexdigest()
+                key = hashlib.sha256(" ".join(flags).encode() + b"".join(f.read_bytes() for f in _with_includes(src))).hexdigest()
                 keyfile = out / (src.stem + ".key")
                 if object_dir and obj.exists() and keyfile.exists() and keyfile.read_text() == key:
                     continue

@@ -23,6 +23,15 @@ constexpr uint32_t kQNaN = 0x7fc00000u;
 __device__ __forceinline__ uint32_t f2u(float x) { return __float_as_uint(x); }
 __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 
+// The matrix kernels' plain inner loop (integer add of the bit patterns) is exact when every value of a k-tile is a
+// normal number with magnitude in [2^-63, 2^64) -- biased exponent 64 ... 190 -- or a zero, which has loops of its
+// own.  Any other value (subnormal, inf, NaN, an extreme exponent) needs the full definition of the product.
+// The staging classifier, the per-k-step record and the marked k-step of the mixed loop all decide by this.
+__device__ __forceinline__ bool needs_full_definition(uint32_t bits)
+{
+    return (bits & ~kSign) != 0 && ((bits >> 23) & 0xffu) - 64u > 126u;
+}
+
 // Finite non-zero magnitude -> unbiased exponent and 23-bit fraction, subnormals normalised.
 __device__ __forceinline__ void split_mag(uint32_t mag, int& e, uint32_t& m)
 {

@@ -39,7 +39,7 @@ def _unfold(X, case):
 
 
 def _plan(batch, m, n, k):
-    return _abi.gemm_plan(batch, m, n, k)[0]
+    return _abi.gemm_plan(batch, m, n, k)
 
 
 @pytest.mark.parametrize("off", [None, OFF])

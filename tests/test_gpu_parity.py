@@ -43,8 +43,8 @@ def ogemm(oracle, L, R, plan_shape=None, **kw):
     from pam_amd import _abi
     L = np.asarray(L); R = np.asarray(R)
     batch = L.shape[0] if L.ndim == 3 else 1
-    chunk, group = _abi.gemm_plan(*(plan_shape or (batch, L.shape[-2], R.shape[-1], L.shape[-1])))
-    return oracle.gemm(L, R, kchunk=chunk, kgroup=group, **kw)
+    chunk = _abi.gemm_plan(*(plan_shape or (batch, L.shape[-2], R.shape[-1], L.shape[-1])))
+    return oracle.gemm(L, R, kchunk=chunk, **kw)
 
 
 def _o(off):
@@ -350,13 +350,16 @@ def test_bmm_tails_and_strides(K, oracle):
 def test_split_k_fixed_order(K, oracle):
     from pam_amd import _abi
     m, n, k = 96, 160, 8192
-    chunk, group = _abi.gemm_plan(1, m, n, k)
-    assert chunk % 16 == 0 and chunk * group < k, "this shape is expected to split k across work-groups"
+    chunk = _abi.gemm_plan(1, m, n, k)
+    assert chunk % 16 == 0 and chunk < k, "this shape is expected to split k across work-groups"
     A, B = _rand((m, k), 14), _rand((k, n), 15)
-    want = oracle.gemm(A, B, kchunk=chunk, kgroup=group)
+    want = oracle.gemm(A, B, kchunk=chunk)
     assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)), want, "split-K order")
     At = dev(np.ascontiguousarray(A.T)).T                      # the dW layout: column-major left operand
     assert_same_bits(host(K.pam_matmul_fwd(At, dev(B), False, True, 1.0)), want, "split-K, cm x rm")
+    # the same call again and again finds the queue and arrival words as the call before left them
+    for _ in range(3):
+        assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0)), want, "repeated call")
     # the sequential order differs from the split order only by fp32 rounding of the sums
     seq = oracle.gemm(A, B)
     assert np.abs(seq - want).max() <= 1e-5 * np.abs(seq).max()
