@@ -121,17 +121,18 @@ def gemm_plan(batch, m, n, k):
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
-# The matrix products' scratch (queue words, pieces of cut tiles): one buffer per device and stream, kept and grown
-# as needed -- products on one stream run one after the other and each leaves the buffer ready for the next, and the
-# buffer is never handed to anything else, so its words are always either fresh zeros or what a product left.
+# The matrix products' scratch (pieces of cut tiles, their arrival words): one buffer per device and stream, kept and
+# grown as needed.  Products on one stream run one after the other, and each leaves the arrival words ready for the
+# next one; products on different streams may overlap in time and must not share a buffer.
 _workspaces = {}
 
 
 def _gemm_workspace(device, nbytes):
-    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    """Called with `device` current."""
+    key = (device.index, _stream())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() * 4 < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20) // 4 + 64, dtype=torch.float32, device=device)
+        ws = torch.empty(max(nbytes, 1 << 20) // 4 + 64, dtype=torch.float32, device=device)
         _workspaces[key] = ws
     return ws
 
@@ -573,7 +574,7 @@ def linear_fwd(X, Wt, bias, offset):
     if out.numel():
         with _on(X.device):
             ws_bytes = load_library().pam_hip_gemm_workspace_bytes(1, m, n, k)
-            ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
+            ws = _gemm_workspace(X.device, ws_bytes) if ws_bytes else None
             _call("pam_hip_pam_linear_fwd", X.data_ptr(), X.stride(0), X.stride(1), Wt.data_ptr(), Wt.stride(0), Wt.stride(1),
                   None if bias is None else bias.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), m, n, k,
                   float(offset), ws.data_ptr() if ws is not None else None, ws_bytes, _stream())

@@ -38,6 +38,7 @@ struct Plan { int bk, kt, pieces, piece_kt; long units; };
 // pieces 0 = automatic, > 0 that many k ranges per tile (as far as k allows).
 thread_local int g_force_bk = 0, g_force_pieces = 0;
 
+constexpr long kMostCutTiles = 8192;            // tiles of a product that cuts them (its arrival words: 64 KB)
 constexpr int kResidentPerCu = 4;               // work-groups of the kernel a compute unit holds (LDS and registers)
 constexpr size_t kPartBytes = (size_t)pamgemm::kPartFloats * sizeof(float);
 
@@ -61,7 +62,7 @@ Plan make_plan(long batch, long M, long N, long K, bool with_workspace)
     const long most = p.kt / least;                                   // pieces a tile can be cut into
     long want = 1;
     if (g_force_pieces > 0) want = g_force_pieces;
-    else if (tiles < (3 * resident) / 2 && with_workspace) {
+    else if (tiles < (3 * resident) / 2 && tiles <= kMostCutTiles && with_workspace) {
         // Time of the product cut into w pieces, in k-tile times of a work-group alone on its compute unit; fitted to
         // measurements on the 12608 x 192 <-> 768 products.  A unit costs its k-tiles plus about one more (fetch of its
         // first k-tile, way out, arrival).  Up to one unit per compute unit they all run at that speed; four on a compute
@@ -81,7 +82,7 @@ Plan make_plan(long batch, long M, long N, long K, bool with_workspace)
         }
     }
     if (want > most) want = most;
-    if (with_workspace && want > 1 && tiles * want < (1L << 31) - 64) {
+    if (with_workspace && want > 1 && tiles <= kMostCutTiles) {
         p.piece_kt = (int)((p.kt + want - 1) / want);
         p.pieces = (p.kt + p.piece_kt - 1) / p.piece_kt;
     }
@@ -89,13 +90,16 @@ Plan make_plan(long batch, long M, long N, long K, bool with_workspace)
     return p;
 }
 
-// workspace of a plan that cuts tiles: [one arrival word per tile][one piece per unit]
+// workspace of a plan that cuts tiles: [arrival words, one per tile][one piece per unit].  The words' part has one size
+// for every shape, so that products of different shapes that share a workspace never write pieces over each other's
+// words (a word that does not carry the launch's tag costs its first arriver two more round trips).
+constexpr size_t kArriveBytes = (size_t)kMostCutTiles * sizeof(unsigned long long);
 struct Space { size_t partial, total; };
 Space plan_space(const Plan& p)
 {
     Space w{0, 0};
     if (p.pieces > 1) {
-        w.partial = ((size_t)(p.units / p.pieces) * sizeof(unsigned long long) + 255) & ~(size_t)255;
+        w.partial = kArriveBytes;
         w.total = w.partial + (size_t)p.units * kPartBytes;
     }
     return w;

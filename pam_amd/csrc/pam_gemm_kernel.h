@@ -584,19 +584,19 @@ __device__ __forceinline__ void pam_bwd_mac_4x4(float (&acc)[4][4], const uint32
 constexpr int kTagShift = 24;                                       // a word: 40 bits of tag, 24 bits of arrivals
 constexpr unsigned long long kTagMask = (1ull << 40) - 1;
 
-// An arrival at a word that carries another tag: whoever exchanges it for one with this launch's tag first is arrival
-// 0, the others (whose adds went to the old contents and are lost with them) arrive again.  Each round ends with
-// some work-group's progress, and there are no more rounds than pieces.
-__device__ __forceinline__ uint32_t arrive_untagged(unsigned long long* word, unsigned long long tag)
+// An arrival at a word that carries another tag (`seen`: what it held after this work-group's add): whoever exchanges
+// it for one with this launch's tag first is arrival 0, the others (whose adds went to the old contents and are lost
+// with them) arrive again.  Each round ends with some work-group's progress, and there are no more rounds than pieces.
+__device__ __forceinline__ uint32_t arrive_untagged(unsigned long long* word, unsigned long long tag, unsigned long long seen)
 {
     for (;;) {
-        unsigned long long seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if ((seen >> kTagShift) == tag) {
             seen = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if ((seen >> kTagShift) == tag) return (uint32_t)(seen & ((1u << kTagShift) - 1));
+            seen += 1ull;
         } else if (__hip_atomic_compare_exchange_strong(word, &seen, (tag << kTagShift) | 1ull, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
             return 0u;
-        }
+        }                                         // (a failed exchange has put the word's present contents into `seen`)
     }
 }
 
@@ -604,7 +604,7 @@ __device__ __forceinline__ uint32_t arrive_untagged(unsigned long long* word, un
 __device__ __forceinline__ uint32_t arrive_at(unsigned long long* word, unsigned long long tag)
 {
     const unsigned long long seen = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return __builtin_expect((seen >> kTagShift) == tag, 1) ? (uint32_t)(seen & ((1u << kTagShift) - 1)) : arrive_untagged(word, tag);
+    return __builtin_expect((seen >> kTagShift) == tag, 1) ? (uint32_t)(seen & ((1u << kTagShift) - 1)) : arrive_untagged(word, tag, seen + 1ull);
 }
 
 constexpr int kPartFloats = 64 * 64;            // one piece of a tile: sixteen sums per lane of the work-group
@@ -653,7 +653,9 @@ __device__ __forceinline__ void fold_pieces(float* partial, long first, int coun
     }
 }
 
-template <int BM, int BN, int TM, int TN, int BK, int MODE, int LKIND, int RKIND>
+// CUT: the launch cuts its tiles' k ranges into pieces (an instance of its own, so that the kernel for whole tiles
+// carries none of the pieces' way out).
+template <int BM, int BN, int TM, int TN, int BK, int MODE, int LKIND, int RKIND, bool CUT>
 __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm_kernel(GemmArgs g)
 {
     constexpr int TXN = BN / TN, TYN = BM / TM, NT = TXN * TYN, NW = NT / 64;
@@ -677,11 +679,18 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         unit = (int)(blockIdx.x % XCDS) * g.xcd_chunk + (int)(blockIdx.x / XCDS);
         if (unit >= g.units) return;              // the ranges are rounded up: a few work-groups have nothing to do
     }
-    const int flat = unit / g.pieces, piece = unit - flat * g.pieces;       // tile of all matrices, k range of it
+    // The unit's tile (of all matrices) and k range.  Tiles cut into few pieces: a tile's pieces are consecutive units, so
+    // they finish at about the same time and the tile is added up early.  Many pieces (few tiles, the weight-gradient
+    // shape): the tiles of one k range are consecutive units -- they run together and share its rows of both operands.
+    int flat = unit, piece = 0;
+    if (CUT) {
+        if (g.fold_here) { flat = unit / g.pieces; piece = unit - flat * g.pieces; }
+        else { const int all = g.units / g.pieces; piece = unit / all; flat = unit - piece * all; }
+    }
     const int zb = flat / g.tiles, tile = flat - zb * g.tiles;
     const int row0 = (tile / g.ntn) * BM, col0 = (tile % g.ntn) * BN;       // consecutive tiles share L rows
-    const int kbegin = piece * g.piece_kt * BK;
-    const int kend = min(g.K, kbegin + g.piece_kt * BK);
+    const int kbegin = CUT ? piece * g.piece_kt * BK : 0;
+    const int kend = CUT ? min(g.K, kbegin + g.piece_kt * BK) : g.K;
     const int ktiles = (kend - kbegin + BK - 1) / BK;
     const bool has_off = g.has_off != 0;
 
@@ -1058,10 +1067,10 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     // ---- the sums' way out
     // A piece of a cut tile goes to its slot of the workspace.  If that completes the tile (and the launch folds its
     // tiles itself), the pieces are added in ascending k order from +0.
-    if (g.pieces > 1) {
+    if constexpr (CUT) {
         if (!g.fold_here) {                       // a second kernel adds the pieces: ordinary stores, the launch's end publishes them
 #pragma unroll
-            for (int i = 0; i < TM; ++i) *piece_row(g.partial, unit, i, tid) = v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+            for (int i = 0; i < TM; ++i) *piece_row(g.partial, (long)flat * g.pieces + piece, i, tid) = v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
             return;
         }
 #pragma unroll
@@ -1118,7 +1127,11 @@ template <int BK, int MODE>
 void launch_gemm(int lk, int rk, unsigned groups, hipStream_t st, const GemmArgs& g)
 {
 #define PAM_GEMM_CASE(LK, RK) \
-    if (lk == LK && rk == RK) { hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 4, BK, MODE, LK, RK>), dim3(groups), dim3(256), 0, st, g); return; }
+    if (lk == LK && rk == RK) {                                                                                                   \
+        if (g.pieces > 1) hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 4, BK, MODE, LK, RK, true>), dim3(groups), dim3(256), 0, st, g);  \
+        else hipLaunchKernelGGL((gemm_kernel<64, 64, 4, 4, BK, MODE, LK, RK, false>), dim3(groups), dim3(256), 0, st, g);            \
+        return;                                                                                                                   \
+    }
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_KVEC, LOAD_RVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_RVEC)
     PAM_GEMM_CASE(LOAD_KVEC, LOAD_ANY)
     PAM_GEMM_CASE(LOAD_RVEC, LOAD_KVEC) PAM_GEMM_CASE(LOAD_RVEC, LOAD_ANY)
