@@ -156,6 +156,14 @@ constexpr uint32_t kIdle = 8u;
 constexpr uint32_t kStandInL = 63u << 23;
 constexpr uint32_t kStandInR = 64u << 23;
 
+// Where row `row` of k-step `k` sits within the k-step's line of a staged tile.  A 32-deep tile's lines 16 ... 31 have
+// their 8-row groups exchanged in pairs (row ^ 8): the transposing writes of an operand whose contiguous dimension is k
+// put a wavefront's eight k-quads at line distances that are multiples of 16 x (64 + 4) words = 0 mod 64 banks, so quads
+// q and q + 4 would meet in the same banks; with the exchange they do not, and groups of four rows stay together for the
+// 128-bit reads.
+template <int BK>
+__device__ __forceinline__ int swizzled(int row, int k) { return BK == 32 ? row ^ ((k & 16) >> 1) : row; }
+
 // One operand's tile: ROWS x BK values from global memory into registers, then into LDS.
 template <int ROWS, int NT, int KIND, int BK>
 struct TileLoader {
@@ -283,7 +291,7 @@ struct TileLoader {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
-                uint32_t* d = lds + ((id % (BK / 4)) * 4) * LD + id / (BK / 4);
+                uint32_t* d = lds + ((id % (BK / 4)) * 4) * LD + swizzled<BK>(id / (BK / 4), (id % (BK / 4)) * 4);
                 d[0 * LD] = st.one(v[i].x); d[1 * LD] = st.one(v[i].y);
                 d[2 * LD] = st.one(v[i].z); d[3 * LD] = st.one(v[i].w);
             }
@@ -293,14 +301,14 @@ struct TileLoader {
                 int id = tid + i * NT;
                 uint4 w;
                 w.x = st.one(v[i].x); w.y = st.one(v[i].y); w.z = st.one(v[i].z); w.w = st.one(v[i].w);
-                *reinterpret_cast<uint4*>(lds + (id / (ROWS / 4)) * LD + (id % (ROWS / 4)) * 4) = w;
+                *reinterpret_cast<uint4*>(lds + (id / (ROWS / 4)) * LD + swizzled<BK>((id % (ROWS / 4)) * 4, id / (ROWS / 4))) = w;
             }
         } else {                                    // LOAD_ANY and LOAD_CONV: lane-consecutive rows
             const float* s = reinterpret_cast<const float*>(v);
 #pragma unroll
             for (int i = 0; i < kElems; ++i) {
                 int id = tid + i * NT;
-                lds[(id / ROWS) * LD + id % ROWS] = st.one(s[i]);
+                lds[(id / ROWS) * LD + swizzled<BK>(id % ROWS, id / ROWS)] = st.one(s[i]);
             }
         }
     }
@@ -769,7 +777,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     __syncthreads();
 
     // per k-tile: where its fragments are in LDS, how many k it holds, and what the staging found in it
-    const uint32_t* sl = nullptr; const uint32_t* sr = nullptr;
+    const uint32_t* sl = nullptr; const uint32_t* sr = nullptr;           // the lane's rows of k-steps 0 ... 15
+    const uint32_t* slx = nullptr; const uint32_t* srx = nullptr;         // and of k-steps 16 ... 31 (see swizzled)
     int kcount = 0;
     const bool idle_wave = MODE != MODE_STD && __builtin_amdgcn_readfirstlane(row0 + (wave * 64 / TXN) * 4 >= g.M ? 1 : 0) != 0;
     uint32_t verdict = 0;                         // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
@@ -788,8 +797,8 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             for (int w = 0; w < NW; ++w) f |= lds_flag[cur][w];
             verdict = idle_wave ? kIdle : __builtin_amdgcn_readfirstlane(f);
         }
-        sl = lds_l[cur] + ty * 4;
-        sr = lds_r[cur] + tx * 4;
+        sl = lds_l[cur] + ty * 4; slx = lds_l[cur] + swizzled<BK>(ty * 4, 16);
+        sr = lds_r[cur] + tx * 4; srx = lds_r[cur] + swizzled<BK>(tx * 4, 16);
     };
     auto end_tile = [&](int t) __attribute__((always_inline)) {
         if (t + 1 < ktiles) stage((t & 1) ^ 1);
@@ -799,12 +808,12 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     auto fragment = [&](int kk, uint32_t (&a)[TM], uint32_t (&b)[TN]) __attribute__((always_inline)) {
 #pragma unroll
         for (int gi = 0; gi < GM; ++gi) {
-            uint4 q = *reinterpret_cast<const uint4*>(sl + kk * LDL + gi * (BM / GM));
+            uint4 q = *reinterpret_cast<const uint4*>(((BK == 32 && (kk & 16)) ? slx : sl) + kk * LDL + gi * (BM / GM));
             a[gi * 4 + 0] = q.x; a[gi * 4 + 1] = q.y; a[gi * 4 + 2] = q.z; a[gi * 4 + 3] = q.w;
         }
 #pragma unroll
         for (int gj = 0; gj < GN; ++gj) {
-            uint4 q = *reinterpret_cast<const uint4*>(sr + kk * LDR + gj * (BN / GN));
+            uint4 q = *reinterpret_cast<const uint4*>(((BK == 32 && (kk & 16)) ? srx : sr) + kk * LDR + gj * (BN / GN));
             b[gj * 4 + 0] = q.x; b[gj * 4 + 1] = q.y; b[gj * 4 + 2] = q.z; b[gj * 4 + 3] = q.w;
         }
     };
@@ -903,14 +912,16 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         if constexpr (MODE != MODE_STD && TM == 4 && TN == 4) {
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            uint32_t plx = (uint32_t)(uintptr_t)(LdsWord)slx, prx = (uint32_t)(uintptr_t)(LdsWord)srx;
             u32x4 fa[2], fb[2];
             fa[0] = *reinterpret_cast<LdsVec>(pl); fb[0] = *reinterpret_cast<LdsVec>(pr);
 #pragma unroll
             for (int kk = 0; kk < BK; ++kk) {
                 if (kk + 1 < BK) {
-                    fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
-                    fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
+                    fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>((kk + 1 < 16 ? pl : plx) + (kk + 1) * LDL * 4);
+                    fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>((kk + 1 < 16 ? pr : prx) + (kk + 1) * LDR * 4);
                 }
+                asm volatile("" : "+v"(plx), "+v"(prx));         // (the blocks below hold the other two addresses the same way)
                 if constexpr (MODE == MODE_PAM) pam_mac_4x4(acc, fa[kk & 1], fb[kk & 1], pl, pr);
                 else pam_bwd_mac_4x4<MODE == MODE_BWD_DL>(acc, dfrac, fa[kk & 1], fb[kk & 1], pl, pr);
             }
@@ -921,13 +932,14 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             static_assert(TM == 4 && TN == 4, "the step fence names sixteen accumulators");
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            uint32_t plx = (uint32_t)(uintptr_t)(LdsWord)slx, prx = (uint32_t)(uintptr_t)(LdsWord)srx;
             u32x4 va[2], vb[2];
             va[0] = *reinterpret_cast<LdsVec>(pl); vb[0] = *reinterpret_cast<LdsVec>(pr);
 #pragma unroll
             for (int kk = 0; kk < BK; ++kk) {
                 if (kk + 1 < BK) {
-                    va[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
-                    vb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
+                    va[(kk + 1) & 1] = *reinterpret_cast<LdsVec>((kk + 1 < 16 ? pl : plx) + (kk + 1) * LDL * 4);
+                    vb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>((kk + 1 < 16 ? pr : prx) + (kk + 1) * LDR * 4);
                 }
                 const uint32_t fa[4] = {va[kk & 1].x, va[kk & 1].y, va[kk & 1].z, va[kk & 1].w};
                 const uint32_t fb[4] = {vb[kk & 1].x, vb[kk & 1].y, vb[kk & 1].z, vb[kk & 1].w};
@@ -940,7 +952,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                         else if (MODE == MODE_BWD_DL) acc[i][j] = fmaf(u2f(fa[i]), u2f((fb[j] + dfrac[i][j]) & ~kMant), acc[i][j]);
                         else acc[i][j] = fmaf(u2f(fb[j]), u2f((fa[i] + dfrac[i][j]) & ~kMant), acc[i][j]);
                     }
-                asm volatile("" : "+v"(pl), "+v"(pr),
+                asm volatile("" : "+v"(pl), "+v"(pr), "+v"(plx), "+v"(prx),
                              "+v"(acc[0][0]), "+v"(acc[0][1]), "+v"(acc[0][2]), "+v"(acc[0][3]), "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]), "+v"(acc[1][3]),
                              "+v"(acc[2][0]), "+v"(acc[2][1]), "+v"(acc[2][2]), "+v"(acc[2][3]), "+v"(acc[3][0]), "+v"(acc[3][1]), "+v"(acc[3][2]), "+v"(acc[3][3]));
             }
@@ -952,14 +964,16 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         if constexpr (MODE == MODE_PAM && TM == 4 && TN == 4) {
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            uint32_t plx = (uint32_t)(uintptr_t)(LdsWord)slx, prx = (uint32_t)(uintptr_t)(LdsWord)srx;
             u32x4 fa[2], fb[2];
             fa[0] = *reinterpret_cast<LdsVec>(pl); fb[0] = *reinterpret_cast<LdsVec>(pr);
 #pragma unroll
             for (int kk = 0; kk < BK; ++kk) {
                 if (kk + 1 < BK) {
-                    fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pl + (kk + 1) * LDL * 4);
-                    fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>(pr + (kk + 1) * LDR * 4);
+                    fa[(kk + 1) & 1] = *reinterpret_cast<LdsVec>((kk + 1 < 16 ? pl : plx) + (kk + 1) * LDL * 4);
+                    fb[(kk + 1) & 1] = *reinterpret_cast<LdsVec>((kk + 1 < 16 ? pr : prx) + (kk + 1) * LDR * 4);
                 }
+                asm volatile("" : "+v"(plx), "+v"(prx));         // (the blocks below hold the other two addresses the same way)
                 constexpr uint32_t kWhich = decltype(which)::value;
                 if constexpr (kWhich == (kZerosL | kZerosR)) pam_mac_4x4_skip_both(acc, fa[kk & 1], fb[kk & 1], pl, pr);
                 else pam_mac_4x4_skip<kWhich == kZerosL>(acc, fa[kk & 1], fb[kk & 1], pl, pr);
@@ -976,8 +990,10 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             constexpr bool ZEROS = decltype(holds_zeros)::value;
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
+            const uint32_t to_plx = (uint32_t)(uintptr_t)(LdsWord)slx - pl, to_prx = (uint32_t)(uintptr_t)(LdsWord)srx - pr;
 #pragma unroll 1
             for (int kk = 0; kk < BK; ++kk) {
+                if (BK == 32 && kk == 16) { pl += to_plx; pr += to_prx; }        // (see swizzled)
                 const u32x4 va = *reinterpret_cast<LdsVec>(pl), vb = *reinterpret_cast<LdsVec>(pr);
                 pl += LDL * 4; pr += LDR * 4;
                 // a marked step concerns the wavefronts whose lanes hold one of its odd values: 16 of a work-group's 256

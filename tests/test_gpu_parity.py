@@ -415,6 +415,18 @@ def test_deit_linear_full_size(K, oracle):
     W2s = (W2 * (rng.rand(*W2.shape) >= 0.3)).astype(np.float32)
     Y2s = K.pam_matmul_fwd(dev(X2r), dev(W2s).T, True, False, 1.0)
     assert_same_bits(host(Y2s)[rows], ogemm(oracle, X2r[rows], W2s.T, plan_shape=(1, 12608, 192, 768)), "Y rows, ReLU input, pruned weight")
+    # the input gradient of the 768 -> 192 layer: row-major times row-major with k = 192
+    dX2 = K.pam_matmul_fwd(dev(dY2), dev(W2), True, True, 1.0)
+    assert_same_bits(host(dX2)[rows], ogemm(oracle, dY2[rows], W2, plan_shape=(1, 12608, 768, 192)), "dX rows, 768 -> 192")
+    # the exact gradients of the 192 -> 768 layer (the calls of pam/cuda_bindings.py:154-164), with and without an offset:
+    # dX = bwd(dY, W, X, delta is the left operand), dW^T = bwd(X^T, dY, W^T, delta is the right operand)
+    for off in OFFS:
+        edX = K.pam_matmul_bwd(tdY, tW, tX, True, True, True, _o(off))
+        assert_same_bits(host(edX)[rows], ogemm(oracle, dY[rows], W, plan_shape=(1, 12608, 192, 768), mode=oracle.MODE_BWD_DELTA_L,
+                                                D=X[rows], offset=off), f"exact dX rows off={off}")
+        edW = K.pam_matmul_bwd(tX.T, tdY, tW.T, False, True, False, _o(off))
+        assert_same_bits(host(edW)[:, cols], ogemm(oracle, X.T, dY[:, cols], plan_shape=(1, 192, 768, 12608), mode=oracle.MODE_BWD_DELTA_R,
+                                                   D=np.ascontiguousarray(W.T[:, cols]), offset=off), f"exact dW cols off={off}")
     # multiplying an operand by a power of two multiplies every PAM product, hence the sum, exactly
     assert torch.equal(K.pam_matmul_fwd(tX * 4.0, tW.T, True, False, 1.0), Y * 4.0)
     assert torch.equal(K.pam_matmul_fwd(tX, (tW * 0.5).T, True, False, 1.0), Y * 0.5)

@@ -38,6 +38,21 @@ def test_noalloc_matches_workspace_variant_twice():
     assert np.array_equal(want.view(np.uint32), got.view(np.uint32))
 
 
+def test_noalloc_call_allocates_nothing():
+    """Device memory in use is the same before and after a call (the first call on a device has looked up the scratch
+    array's address by then, which may load the code object: callers under graph capture make one call beforehand)."""
+    from pam_amd import _abi
+    m, n, k = 192, 768, 12608
+    g = torch.Generator().manual_seed(5)
+    A = torch.randn(m, k, generator=g).cuda(); B = torch.randn(k, n, generator=g).cuda(); Y = torch.empty(m, n, device="cuda")
+    call = lambda: _abi._call("pam_hip_pam_matmul_fwd_noalloc", A.data_ptr(), k, 1, B.data_ptr(), n, 1, Y.data_ptr(), n, 1, m, n, k, 1.0, _abi._stream())
+    call(); torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info(); held0 = torch.cuda.memory_allocated(); reserved0 = torch.cuda.memory_reserved()
+    call(); call(); torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_allocated() == held0 and torch.cuda.memory_reserved() == reserved0
+
+
 def test_noalloc_refuses_what_does_not_fit():
     from pam_amd import _abi
     lib = _abi.load_library()
