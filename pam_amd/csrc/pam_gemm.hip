@@ -143,7 +143,9 @@ __global__ __launch_bounds__(128) void fold_kernel(pamgemm::GemmArgs g)
     }
     for (; p < g.pieces; ++p) total += *pamgemm::piece_row(g.partial, first + p, i, tid);
     const int zb = flat / g.tiles, tile = flat - zb * g.tiles, tr = tile / g.ntn;
-    const int r = tr * 64 + (tid / 16) * 4 + i, c = (tile - tr * g.ntn) * 64 + (tid % 16) * 4;
+    const int row0 = tr * 64, col0 = (tile - tr * g.ntn) * 64;
+    const pamgemm::LanePlace place = pamgemm::lane_place(tid, row0, col0, g.M, g.N);
+    const int r = row0 + place.ty * 4 + i, c = col0 + place.tx * 4;
     if (r >= g.M) return;
     float* dst = g.Y + (long)zb * g.y_sb + (long)r * g.y_sr + (long)c * g.y_sc;
     const float sums[4] = {total.x, total.y, total.z, total.w};

@@ -145,9 +145,7 @@ __device__ __forceinline__ uint32_t max3u(uint32_t a, uint32_t b, uint32_t c) { 
 // Verdict of a k-tile: bit 0 / bit 1 = the left / right operand holds zeros (all else in range),
 // kGuarded = some value needs the full definition.  Verdicts of wavefronts combine by OR.
 constexpr uint32_t kZerosL = 1u, kZerosR = 2u, kGuarded = 4u;
-// A wavefront all of whose rows lie beyond M (the last row tile of a matrix whose height is not a multiple of the
-// tile: 197 rows leave three of the four wavefronts of the fourth tile without a row) stages and synchronises with
-// the others but computes nothing.
+// A wavefront none of whose outputs exist (see lane_place) stages and synchronises with the others but computes nothing.
 constexpr uint32_t kIdle = 8u;
 
 // Stand-ins that keep the integer sum a finite number when one operand is zero: 2^-64 on the
@@ -620,6 +618,18 @@ constexpr int kFoldInKernel = 8;                // tiles of up to this many piec
 
 // A piece of a cut tile in the workspace: the work-group's lanes' sixteen sums each as four 128-bit rows, row i of
 // lane `tid` at [unit][i][tid] -- every access of the work-group is one contiguous 4 KB run.
+// Where a lane's 4 x 4 outputs sit in its work-group's 64 x 64 tile: rows ty * 4 ..., columns tx * 4 ....  A wavefront
+// covers 16 rows x 64 columns -- or, in a tile that the matrix fills less in its columns than in its rows, 64 rows x
+// 16 columns: a wavefront none of whose outputs exist (the last tiles of 197 rows or columns leave three of the four
+// without one) stages and synchronises with the others but computes nothing.
+struct LanePlace { int tx, ty; bool idle; };
+__device__ __forceinline__ LanePlace lane_place(int tid, int row0, int col0, int M, int N)
+{
+    const int wave = tid / 64, lane = tid % 64;
+    if (N - col0 < 64 && N - col0 < M - row0) return LanePlace{4 * wave + lane % 4, lane / 4, col0 + 16 * wave >= N};
+    return LanePlace{tid % 16, tid / 16, row0 + 16 * wave >= M};
+}
+
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned long long Pair;                // half a row, where the access has to be an atomic one
 __device__ __forceinline__ v4f* piece_row(float* partial, long unit, int i, int tid)
@@ -677,7 +687,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     __shared__ uint32_t lds_odd_k[2][NW];         // bit k: some value under k of the tile needs the full definition
     __shared__ uint32_t lds_arrived;
 
-    const int tid = threadIdx.x, tx = tid % TXN, ty = tid / TXN;
+    const int tid = threadIdx.x;
     const int wave = tid / 64, lane = tid % 64;
     // This work-group's unit.  Work-groups go to the eight XCDs in turn and every XCD has its own L2, so with units in
     // launch order the column tiles of one row tile land on all eight and each L2 fetches the whole left operand.
@@ -700,6 +710,9 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     const int kbegin = CUT ? piece * g.piece_kt * BK : 0;
     const int kend = CUT ? min(g.K, kbegin + g.piece_kt * BK) : g.K;
     const int ktiles = (kend - kbegin + BK - 1) / BK;
+    // The lane's 4 x 4 outputs within the tile, rows ty * 4 ..., columns tx * 4 ....
+    const LanePlace place = lane_place(tid, row0, col0, g.M, g.N);
+    const int tx = place.tx, ty = place.ty;
     const bool has_off = g.has_off != 0;
 
     const float* lbase = g.L.p + (long)zb * g.L.sb;
@@ -780,7 +793,7 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     const uint32_t* sl = nullptr; const uint32_t* sr = nullptr;           // the lane's rows of k-steps 0 ... 15
     const uint32_t* slx = nullptr; const uint32_t* srx = nullptr;         // and of k-steps 16 ... 31 (see swizzled)
     int kcount = 0;
-    const bool idle_wave = MODE != MODE_STD && __builtin_amdgcn_readfirstlane(row0 + (wave * 64 / TXN) * 4 >= g.M ? 1 : 0) != 0;
+    const bool idle_wave = MODE != MODE_STD && __builtin_amdgcn_readfirstlane(place.idle ? 1 : 0) != 0;
     uint32_t verdict = 0;                         // 0 plain loop, kZerosL / kZerosR bits, >= kGuarded guarded
     auto begin_tile = [&](int t) __attribute__((always_inline)) {
         const int cur = t & 1;
