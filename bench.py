@@ -33,10 +33,61 @@ def parse():
     ap.add_argument("--no-elementwise", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one device-to-device copy of 2^26 floats (calibrates FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--write-traffic", metavar="DIR",
+                    help="no GPU work: read the FETCH_SIZE and WRITE_SIZE counter passes of this program under DIR "
+                         "(DIR/pmc_<COUNTER>/p_counter_collection.csv, DIR/pmc_<COUNTER>.json = that pass's bench line) "
+                         "and rewrite profiles/traffic.json, stamped with the source hash of the library they measured")
     return ap.parse_args()
 
 
 SETTLE_S = 0.03
+HERE = os.path.dirname(os.path.abspath(__file__))
+TRAFFIC_FILE = os.path.join(HERE, "profiles", "traffic.json")
+HEADLINE_KERNEL = "gemm_kernel<64, 64, 4, 4, 32, 0, 0, 0, false>"      # whole tiles, both operands contiguous along k
+ELEMENTWISE_KERNEL = "ew_vec_kernel<OpPam, 2>"
+
+
+def write_traffic(prof_dir):
+    """HBM bytes per launch of the headline product (12608x768, k = 192) and of the elementwise multiply on 2^26 elements
+    from two counter passes over `bench.py --steps 5 --warmup 2 --no-cpu-baseline --copy-probe --settle-ms 0`.  The
+    counters' unit is calibrated on the elementwise multiply, which reads exactly 2 x 256 MiB and writes 256 MiB."""
+    import csv
+    import re
+    per_counter, stamps = {}, set()
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        with open(os.path.join(prof_dir, f"pmc_{counter}.json")) as f:
+            stamps.add(json.loads(f.read().strip().splitlines()[-1])["library_source_hash"])
+        dispatches = {}
+        with open(os.path.join(prof_dir, f"pmc_{counter}", "p_counter_collection.csv")) as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] != counter:
+                    continue
+                name = re.sub(r"\(anonymous namespace\)::|pamgemm::|^void ", "", r["Kernel_Name"])
+                name = re.sub(r"\(.*", "", name)
+                dispatches[int(r["Dispatch_Id"])] = (name, int(r["Grid_Size"]), float(r["Counter_Value"]))
+        ids = sorted(dispatches)
+        first_ew = min(i for i in ids if dispatches[i][0] == ELEMENTWISE_KERNEL)
+        # the headline product's launches are those of its kernel instance before the first elementwise launch with the
+        # launch size that occurs most often there (the six-product step and the per-product rows)
+        head = [dispatches[i] for i in ids if i < first_ew and dispatches[i][0] == HEADLINE_KERNEL]
+        grids = [g for _, g, _ in head]
+        grid = max(set(grids), key=grids.count)
+        ew = [v for n, g, v in dispatches.values() if n == ELEMENTWISE_KERNEL]
+        per_counter[counter] = (sum(v for _, g, v in head if g == grid) / grids.count(grid), sum(ew) / len(ew))
+    if len(stamps) != 1:
+        sys.exit(f"bench.py: the two counter passes ran different libraries: {sorted(stamps)}")
+    n = 1 << 26
+    known = {"FETCH_SIZE": 8 * n, "WRITE_SIZE": 4 * n}
+    head_bytes = sum(per_counter[c][0] * known[c] / per_counter[c][1] for c in known)
+    out = {"library_source_hash": stamps.pop(), "gemm_fwd_12608x768x192_bytes": round(head_bytes), "ew_mul_2p26_bytes": 12 * n,
+           "counter_units": {c: round(known[c] / per_counter[c][1], 2) for c in known},
+           "source": "FETCH_SIZE and WRITE_SIZE per dispatch (rocprofv3 --pmc over bench.py), in units of what the same counter "
+                     "reads for the elementwise multiply on 2^26 elements (8 and 4 bytes per element); "
+                     "written by bench.py --write-traffic"}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(out, f, indent=1)
+        f.write("\n")
+    print(json.dumps(out))
 
 
 def event_time_ms(fn, iters, torch, settle_s=None):
@@ -88,6 +139,8 @@ def main():
     global SETTLE_S
     args = parse()
     SETTLE_S = args.settle_ms / 1e3
+    if args.write_traffic:
+        return write_traffic(args.write_traffic)
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus must be 1 "
                  "(the path has no collective: it shards by rows, with one all-reduce of dW per layer)")
@@ -172,14 +225,16 @@ def main():
     roofline["register_only_probe_Tlaneop_s"] = {str(w): round(_abi.issue_probe(w), 2) for w in (1, 2, 4, 8)}
     # and with every step's operands read from LDS the way the kernel's inner loop reads them (4 x 4 per lane)
     roofline["lds_fed_4x4_probe_Tlaneop_s"] = {str(w): round(_abi.issue_probe(w, lds_tile=(4, 4)), 2) for w in (1, 2, 4, 8)}
-    traffic_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
-    traffic = json.load(open(traffic_file)) if os.path.exists(traffic_file) else {}
+    # counter-measured HBM bytes per launch, valid only for the library they were measured with
+    traffic = json.load(open(TRAFFIC_FILE)) if os.path.exists(TRAFFIC_FILE) else {}
+    if traffic.get("library_source_hash") != source_stamp:
+        traffic = {}
     roofline["traffic"] = traffic.get("gemm_fwd_12608x768x192_bytes")
 
     # the headline metric as BASELINE.json words it (value = its G-MAC/s part, at the 12608x192x768 configuration;
     # the %VALU-peak part is roofline.frac, the elementwise GB/s part roofline_elementwise.achieved)
     metric_name = "PAM-GEMM G-MAC/s + %VALU peak at 12608x192x768 fp32; PAM elementwise GB/s"
-    baseline_file = os.path.join(os.path.dirname(os.path.abspath(__file__)), "BASELINE.json")
+    baseline_file = os.path.join(HERE, "BASELINE.json")
     if os.path.exists(baseline_file):
         metric_name = json.load(open(baseline_file)).get("metric") or metric_name
     out = {

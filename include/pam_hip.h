@@ -119,7 +119,7 @@ int pam_hip_pam_matmul_fwd(const float *a, long a_sr, long a_sc, const float *b,
  * a workspace of pam_hip_gemm_workspace_bytes(1, m, n, k).  A shape that needs more scratch than the array is
  * refused with PAM_HIP_ERR_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on the
  * same GPU (different streams or threads) race, so serialise them. */
-#define PAM_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+#define PAM_HIP_NOALLOC_SCRATCH_BYTES (48u << 20)
 int pam_hip_pam_matmul_fwd_noalloc(const float *a, long a_sr, long a_sc, const float *b, long b_sr, long b_sc,
                                    float *y, long y_sr, long y_sc, long m, long n, long k, float offset, void *stream);
 /* Y = A (x) B + bias[column]: the product followed by the bias add of pam.linear

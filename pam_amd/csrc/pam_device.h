@@ -27,10 +27,23 @@ __device__ __forceinline__ float u2f(uint32_t u) { return __uint_as_float(u); }
 // normal number with magnitude in [2^-63, 2^64) -- biased exponent 64 ... 190 -- or a zero, which has loops of its
 // own.  Any other value (subnormal, inf, NaN, an extreme exponent) needs the full definition of the product.
 // The staging classifier, the per-k-step record and the marked k-step of the mixed loop all decide by this.
+constexpr uint32_t kPlainExpMin = 64u, kPlainExpMax = 190u;
 __device__ __forceinline__ bool needs_full_definition(uint32_t bits)
 {
-    return (bits & ~kSign) != 0 && ((bits >> 23) & 0xffu) - 64u > 126u;
+    return (bits & ~kSign) != 0 && ((bits >> 23) & 0xffu) - kPlainExpMin > kPlainExpMax - kPlainExpMin;
 }
+// The same predicate over many values at two instructions each: the biased exponents of the values (a zero counts as
+// 127) folded by min and max, compared once at the end.  The staging classifier sees sixteen values per lane and
+// k-tile; the predicate per value cost the convolutions, whose padding sends nearly every k-tile through it, 8 %.
+struct ExponentRange {
+    uint32_t emin = 255u, emax = 0u;
+    __device__ __forceinline__ void see(uint32_t bits, bool is_zero)
+    {
+        const uint32_t e = is_zero ? 127u : (bits >> 23) & 0xffu;
+        emin = min(emin, e); emax = max(emax, e);
+    }
+    __device__ __forceinline__ bool needs_full_definition() const { return emin < kPlainExpMin || emax > kPlainExpMax; }
+};
 
 // Finite non-zero magnitude -> unbiased exponent and 23-bit fraction, subnormals normalised.
 __device__ __forceinline__ void split_mag(uint32_t mag, int& e, uint32_t& m)

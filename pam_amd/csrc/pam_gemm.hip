@@ -46,9 +46,9 @@ constexpr size_t kPartBytes = (size_t)pamgemm::kPartFloats * sizeof(float);
 // from 512, uses 32-deep k-tiles (fewer barriers and more bytes in flight per round, measured 3-5 %
 // faster on 12608-row products); short or ragged k (attention: 64, 197) 16-deep ones.
 // Shapes with few output tiles and long k (dX: 12608 x 192, k = 768; dW: 192 x 768, k = 12608) cut every tile's k
-// range into equal pieces, each at least 128 deep in k, so that the units fill the work-groups the device keeps
-// resident (four per compute unit) about twice over: of the piece counts near that, the one whose last round of
-// resident work-groups is fullest.
+// range into equal pieces, each at least 128 deep in k: few pieces by the cost model below (the tile's last
+// work-group adds them up), or, where that asks for more than a work-group should add up, about two resident rounds of
+// piece-major units and a second kernel.
 Plan make_plan(long batch, long M, long N, long K, bool with_workspace)
 {
     const long resident = (long)kResidentPerCu * cu_count();
@@ -79,6 +79,16 @@ Plan make_plan(long batch, long M, long N, long K, bool with_workspace)
                                                                  : 1.5 * (rounds + 0.15 * (std::ceil(rounds) - rounds));
             const double time = (double)(per + 1) * crowd * (pieces > pamgemm::kFoldInKernel ? 1.03 : 1.0);
             if (best == 0.0 || time < best) { best = time; want = pieces; }
+        }
+        // More pieces than a tile's last work-group adds up itself (few tiles, very long k: the weight gradients): the
+        // units are piece-major and a second kernel adds them.  Measured on 192 x 768, k = 12608, dense and with the
+        // zeros of a ReLU in the left operand, such a launch does best with about two resident rounds of shorter units
+        // in launch order (57 pieces: 86 / 102 us; one round of 27: 88 / 111 us).
+        if (want > pamgemm::kFoldInKernel) {
+            const long target = (2 * resident + tiles - 1) / tiles;
+            long per = (p.kt + target / 2) / target;
+            if (per < least) per = least;
+            want = (p.kt + per - 1) / per;
         }
     }
     if (want > most) want = most;
@@ -165,10 +175,13 @@ int load_kind(long s_row, long s_k, long s_batch, const float* p, long rows, lon
 template <int MODE>
 void launch_mode(const Plan& p, int lk, int rk, hipStream_t st, const GemmArgs& g)
 {
-    // one contiguous range of units per XCD (see the kernel), rounded up to whole work-groups per XCD
+    // One contiguous range of units per XCD (see the kernel), rounded up to whole work-groups per XCD.  Piece-major
+    // launches keep the launch order: all XCDs then work on the same few k ranges at a time (each L2 fetches them,
+    // from the memory-side cache), where ranges would have every L2 hold three or four k ranges of both operands at
+    // once -- measured 3 % (dense) to 9 % (left operand with zeros) slower.
     GemmArgs ga = g;
     unsigned groups = (unsigned)p.units;
-    if (p.units >= 64) {
+    if (p.units >= 64 && (p.pieces == 1 || g.fold_here)) {
         ga.xcd_chunk = (int)((p.units + XCDS - 1) / XCDS);
         groups = (unsigned)(ga.xcd_chunk * XCDS);
     }

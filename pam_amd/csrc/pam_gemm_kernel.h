@@ -5,17 +5,20 @@
 // multiply-accumulate, one v_add_u32 and one v_add_f32.
 //
 //  * A work-group of four wavefronts owns a 64 x 64 tile of Y.  Each lane owns a 4 x 4
-//    micro-tile in registers, each wavefront 32 x 32 outputs (lanes 8 x 8).  Measured on
+//    micro-tile in registers, each wavefront 16 x 64 outputs (lane_place below).  Measured on
 //    MI355X, a SIMD retires a wave64 VALU instruction every two cycles but one wavefront
 //    issues at most one every four, so several wavefronts per SIMD are needed (four are
-//    resident: 104 registers, 35 KB of LDS per work-group with 32-deep k-tiles); larger
+//    resident: at most 128 registers, 35 KB of LDS per work-group with 32-deep k-tiles); larger
 //    micro-tiles and more resident wavefronts were measured and gained nothing.  Thousands
 //    of equal work-groups per product are what balances the 256 compute units.
 //  * L and R tiles are staged through LDS k-major ([k][row], 4-word row pad), so a fragment
 //    for one k is two ds_read_b128, contiguous (R) or broadcast (L) across the wavefront.
 //    Operands whose contiguous dimension is k (row-major L, "column-major" R) are
 //    transposed on the way in; operands contiguous along the row use 128-bit LDS writes;
-//    anything else goes through a scalar loader.  No transposed copies are made in global
+//    anything else goes through a scalar loader.  In a 32-deep tile the lines k = 16 ... 31
+//    keep their 8-row groups exchanged (row ^ 8, `swizzled`): the transposing writes of the
+//    two k halves then fall into different banks (a third of the bank-conflict cycles of the
+//    plain layout).  No transposed copies are made in global
 //    memory, so the backward products run on the views the autograd layer hands over
 //    (pam/cuda_bindings.py:147-164).
 //  * Global loads for k-tile t+1 are issued before the arithmetic of tile t (register
@@ -39,15 +42,17 @@
 //  * Rows beyond M / N are clamped to the last valid row when loading (their results are
 //    never stored); the k tail runs a shorter loop, padding never enters the arithmetic.
 //  * Shapes with few output tiles and long k (dX: 12608 x 192, k = 768; dW: 192 x 768,
-//    k = 12608) split k across work-groups; the partial tiles go through a scratch buffer
-//    and are added in ascending order by a second kernel.
-//  * The launch is one-dimensional over (matrix, k chunk, tile) units and every XCD (own L2)
+//    k = 12608) cut every tile's k range into pieces, one work-group each; the last
+//    work-group to finish a piece of a tile adds the pieces up and writes the tile ("the
+//    units of a launch" below), a second kernel does where the pieces are many.
+//  * The launch is one-dimensional over the units and every XCD (own L2)
 //    takes one contiguous range of them, so each operand is fetched from memory about once.
 //  * The right operand may be the patches of an image read in place (convolutions), and a
 //    bias may be added to the finished sums (linear layers).
-//  * Accumulation order: every output is summed by one lane per k chunk, k ascending, from
-//    +0 -- with one chunk this is the order of the reference kernel
-//    (pam/cuda_kernels.cu:601, 608-627); pam_hip_gemm_plan reports the chunking.
+//  * Accumulation order: every output is summed by one lane per k chunk (piece), k ascending,
+//    from +0, and the chunks' sums are added in ascending order from +0 -- with one chunk
+//    this is the order of the reference kernel (pam/cuda_kernels.cu:601, 608-627);
+//    pam_hip_gemm_plan reports the chunk length.
 #pragma once
 #include <cmath>
 #include <cstring>
@@ -109,23 +114,25 @@ struct Stager {
     static constexpr bool kDeltaSide = (MODE >= MODE_BWD_DL) && !kSlopeSide;
     static constexpr bool kTakesOffset = (MODE == MODE_PAM && IS_R) || kSlopeSide;
     bool bad = false, zero = false;
+    ExponentRange seen;
     __device__ __forceinline__ uint32_t one(float v)
     {
         uint32_t u = f2u(v);
         if (MODE == MODE_STD) return u;
-        bad |= needs_full_definition(u);
         if (MODE == MODE_PAM) {                    // zeros get their own, cheaper loop
             const bool z = (u & ~kSign) == 0;
             zero |= z;
+            seen.see(u, z);
             return z ? (IS_R ? kZeroR : kZeroL) : (IS_R ? u - kBias : u);
         }
+        bad |= needs_full_definition(u);
         // Backward modes.  The upstream gradient: zero is harmless.  The slope side: a zero needs no care either,
         // (0 + fraction) & ~mantissa is 0 and the fma then adds delta * 0 (delta is finite in the plain loop), which
         // is what the definition gives.
         return u;
     }
     // some staged value lies outside [2^-63, 2^64) or is not a normal number or zero
-    __device__ __forceinline__ bool out_of_range() const { return bad; }
+    __device__ __forceinline__ bool out_of_range() const { return bad || (MODE == MODE_PAM && seen.needs_full_definition()); }
 };
 
 // Staging when the quick test below has passed: every value of the k-tile is a normal number in
@@ -294,20 +301,24 @@ struct TileLoader {
                 d[2 * LD] = st.one(v[i].z); d[3 * LD] = st.one(v[i].w);
             }
         } else if (KIND == LOAD_RVEC) {
+            // (vector i of a lane sits under k = i * kPer + tid / (ROWS / 4), the second term below kPer: which half of a
+            // 32-deep tile that is depends on i alone, so the exchange of the row groups costs nothing per vector)
+            constexpr int kPer = NT / (ROWS / 4);
+            static_assert(16 % kPer == 0, "a lane's vectors must not straddle the tile's k halves");
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
-                int id = tid + i * NT;
                 uint4 w;
                 w.x = st.one(v[i].x); w.y = st.one(v[i].y); w.z = st.one(v[i].z); w.w = st.one(v[i].w);
-                *reinterpret_cast<uint4*>(lds + (id / (ROWS / 4)) * LD + swizzled<BK>((id % (ROWS / 4)) * 4, id / (ROWS / 4))) = w;
+                *reinterpret_cast<uint4*>(lds + (i * kPer + tid / (ROWS / 4)) * LD + swizzled<BK>((tid % (ROWS / 4)) * 4, i * kPer)) = w;
             }
         } else {                                    // LOAD_ANY and LOAD_CONV: lane-consecutive rows
             const float* s = reinterpret_cast<const float*>(v);
+            // (element i of a lane sits under k = i * (NT / ROWS) + tid / ROWS: its half of the tile depends on i alone too)
+            static_assert(16 % (NT / ROWS) == 0, "a lane's elements must not straddle the tile's k halves");
+            const int row = tid % ROWS, kwave = tid / ROWS;
 #pragma unroll
-            for (int i = 0; i < kElems; ++i) {
-                int id = tid + i * NT;
-                lds[(id / ROWS) * LD + swizzled<BK>(id % ROWS, id / ROWS)] = st.one(s[i]);
-            }
+            for (int i = 0; i < kElems; ++i)
+                lds[(i * (NT / ROWS) + kwave) * LD + swizzled<BK>(row, i * (NT / ROWS))] = st.one(s[i]);
         }
     }
 };
@@ -616,8 +627,6 @@ __device__ __forceinline__ uint32_t arrive_at(unsigned long long* word, unsigned
 constexpr int kPartFloats = 64 * 64;            // one piece of a tile: sixteen sums per lane of the work-group
 constexpr int kFoldInKernel = 8;                // tiles of up to this many pieces are added up by their last arriver
 
-// A piece of a cut tile in the workspace: the work-group's lanes' sixteen sums each as four 128-bit rows, row i of
-// lane `tid` at [unit][i][tid] -- every access of the work-group is one contiguous 4 KB run.
 // Where a lane's 4 x 4 outputs sit in its work-group's 64 x 64 tile: rows ty * 4 ..., columns tx * 4 ....  A wavefront
 // covers 16 rows x 64 columns -- or, in a tile that the matrix fills less in its columns than in its rows, 64 rows x
 // 16 columns: a wavefront none of whose outputs exist (the last tiles of 197 rows or columns leave three of the four
@@ -631,10 +640,20 @@ __device__ __forceinline__ LanePlace lane_place(int tid, int row0, int col0, int
 }
 
 typedef float v4f __attribute__((ext_vector_type(4)));
-typedef unsigned long long Pair;                // half a row, where the access has to be an atomic one
+// A piece of a cut tile in the workspace: the work-group's lanes' sixteen sums each as four 128-bit rows, row i of
+// lane `tid` at [unit][i][tid] -- every access of the work-group is one contiguous 4 KB run.
 __device__ __forceinline__ v4f* piece_row(float* partial, long unit, int i, int tid)
 {
     return reinterpret_cast<v4f*>(partial) + ((unit * 4 + i) * 256 + tid);
+}
+// The same where the pieces are exchanged inside the launch, which takes agent-scope accesses of at most 64 bits: half
+// rows, half h of row i of lane `tid` at [unit][i][h][tid], so that every access of a wavefront is one contiguous
+// 512-byte run (as halves of the 128-bit rows above, each store filled half of every 32-byte sector it touched, and
+// the write-through stores counted twice their bytes in memory traffic).
+typedef unsigned long long Pair;
+__device__ __forceinline__ Pair* piece_half(float* partial, long unit, int i, int h, int tid)
+{
+    return reinterpret_cast<Pair*>(partial) + ((unit * 8 + i * 2 + h) * 256 + tid);
 }
 
 // acc = the pieces [first, first + count) of a tile added in ascending order from +0, read at agent scope (their
@@ -654,8 +673,8 @@ __device__ __forceinline__ void fold_pieces(float* partial, long first, int coun
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                v[0][i][h] = __hip_atomic_load(reinterpret_cast<Pair*>(piece_row(partial, first + p, i, tid)) + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                v[1][i][h] = __hip_atomic_load(reinterpret_cast<Pair*>(piece_row(partial, first + second, i, tid)) + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v[0][i][h] = __hip_atomic_load(piece_half(partial, first + p, i, h, tid), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                v[1][i][h] = __hip_atomic_load(piece_half(partial, first + second, i, h, tid), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
@@ -669,6 +688,19 @@ __device__ __forceinline__ void fold_pieces(float* partial, long first, int coun
                 }
         }
     }
+}
+
+// What only the sums' way out needs of the arguments (where the output and the pieces are, the bias, the arrival words)
+// is read there from the kernel's argument segment, through a pointer the compiler cannot see through: held in scalar
+// registers from the kernel's start, as it otherwise arranges, they are eighteen registers too many during the loops,
+// which then spill scalar values into vector lanes (the k-tiles with zeros, which live on execution masks, ran 14 %
+// slower for it, and the image-patch instance spilled vector registers on top).
+typedef const __attribute__((address_space(4))) GemmArgs* LateArgs;
+__device__ __forceinline__ LateArgs late_args()
+{
+    LateArgs p = (LateArgs)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return p;
 }
 
 // CUT: the launch cuts its tiles' k ranges into pieces (an instance of its own, so that the kernel for whole tiles
@@ -1096,39 +1128,40 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     // ---- the sums' way out
     // A piece of a cut tile goes to its slot of the workspace.  If that completes the tile (and the launch folds its
     // tiles itself), the pieces are added in ascending k order from +0.
+    const LateArgs e = late_args();
     if constexpr (CUT) {
-        if (!g.fold_here) {                       // a second kernel adds the pieces: ordinary stores, the launch's end publishes them
+        if (!e->fold_here) {                       // a second kernel adds the pieces: ordinary stores, the launch's end publishes them
 #pragma unroll
-            for (int i = 0; i < TM; ++i) *piece_row(g.partial, (long)flat * g.pieces + piece, i, tid) = v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+            for (int i = 0; i < TM; ++i) *piece_row(e->partial, (long)flat * e->pieces + piece, i, tid) = v4f{acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
             return;
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
-                __hip_atomic_store(reinterpret_cast<Pair*>(piece_row(g.partial, unit, i, tid)) + h, ((Pair)f2u(acc[i][2 * h + 1]) << 32) | f2u(acc[i][2 * h]),
+                __hip_atomic_store(piece_half(e->partial, unit, i, h, tid), ((Pair)f2u(acc[i][2 * h + 1]) << 32) | f2u(acc[i][2 * h]),
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // the stores have completed (they are write-through at this scope) before any lane of the work-group arrives
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        unsigned long long* word = g.arrive + flat;
-        if (tid == 0) lds_arrived = arrive_at(word, g.tag) + 1u;
+        unsigned long long* word = e->arrive + flat;
+        if (tid == 0) lds_arrived = arrive_at(word, e->tag) + 1u;
         __syncthreads();
-        if (__builtin_amdgcn_readfirstlane(lds_arrived) != (uint32_t)g.pieces) return;
+        if (__builtin_amdgcn_readfirstlane(lds_arrived) != (uint32_t)e->pieces) return;
         asm volatile("" ::: "memory");
-        fold_pieces(g.partial, (long)flat * g.pieces, g.pieces, tid, acc);
-        if (tid == 0) __hip_atomic_store(word, ((g.tag + 1) & kTagMask) << kTagShift, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);    // ready for the next launch
+        fold_pieces(e->partial, (long)flat * e->pieces, e->pieces, tid, acc);
+        if (tid == 0) __hip_atomic_store(word, ((e->tag + 1) & kTagMask) << kTagShift, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);    // ready for the next launch
     }
     // the finished sums of the tile to Y (plus the bias, if any)
-    float* out = g.Y + (long)zb * g.y_sb;
-    const long o_sr = g.y_sr, o_sc = g.y_sc;
-    if (g.bias) {
+    float* out = e->Y + (long)zb * e->y_sb;
+    const long o_sr = e->y_sr, o_sc = e->y_sc;
+    if (e->bias) {
 #pragma unroll
         for (int gj = 0; gj < GN; ++gj)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int c = col0 + gj * (BN / GN) + tx * 4 + j;
-                const float bv = c < g.N ? g.bias[c] : 0.0f;
+                const float bv = c < g.N ? e->bias[c] : 0.0f;
 #pragma unroll
                 for (int i = 0; i < TM; ++i) acc[i][gj * 4 + j] = acc[i][gj * 4 + j] + bv;
             }
