@@ -81,17 +81,28 @@ Plan make_plan(long batch, long M, long N, long K, bool with_workspace)
             if (best == 0.0 || time < best) { best = time; want = pieces; }
         }
         // More pieces than a tile's last work-group adds up itself (few tiles, very long k: the weight gradients): the
-        // units are piece-major and a second kernel adds them.  Measured on 192 x 768, k = 12608, dense and with the
-        // zeros of a ReLU in the left operand, such a launch does best with about two resident rounds of shorter units
-        // in launch order (57 pieces: 86 / 102 us; one round of 27: 88 / 111 us).
+        // units are piece-major in launch order and a second kernel adds them.  Two work-groups on a compute unit issue
+        // at nearly the rate of four, and a third adds little, so such a launch runs in rounds of two units per compute
+        // unit: its time goes as (rounds + 0.4) x (k-tiles per piece + 1.25), the 0.4 for the skew with which a round's
+        // units end, the 1.25 for a unit's start and way out.  Fitted on weight gradients of 9 ... 144 tiles with k =
+        // 3152 ... 50432 (pieces of 224 k for the 192 x 768, k = 12608 one: 86 us dense, 102 us with the zeros of a
+        // ReLU in the left operand; one resident round of 27 pieces, a range of them per XCD: 88 and 111 us).
         if (want > pamgemm::kFoldInKernel) {
-            const long target = (2 * resident + tiles - 1) / tiles;
-            long per = (p.kt + target / 2) / target;
-            if (per < least) per = least;
-            want = (p.kt + per - 1) / per;
+            const long quantum = 2 * cus;
+            double least_time = 0.0;
+            for (long per = least;; ++per) {
+                const long pieces = (p.kt + per - 1) / per;
+                if (pieces <= pamgemm::kFoldInKernel) break;
+                if (pieces > most) continue;
+                const long n = tiles * pieces;
+                long rounds = (n - n / 50 + quantum - 1) / quantum;               // (2 % over whole rounds still counts as those)
+                if (rounds < 1) rounds = 1;
+                const double time = ((double)rounds + 0.4) * ((double)per + 1.25);
+                if (least_time == 0.0 || time < least_time) { least_time = time; want = pieces; }
+            }
         }
     }
-    if (want > most) want = most;
+    if (want > (g_force_pieces > 0 ? (long)p.kt : most)) want = g_force_pieces > 0 ? (long)p.kt : most;
     if (with_workspace && want > 1 && tiles <= kMostCutTiles) {
         p.piece_kt = (int)((p.kt + want - 1) / want);
         p.pieces = (p.kt + p.piece_kt - 1) / p.piece_kt;
