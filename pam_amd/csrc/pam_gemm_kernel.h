@@ -1027,31 +1027,62 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     };
     constexpr bool kSkips = MODE == MODE_PAM && TM == 4 && TN == 4;
 
-    // a full k-tile some of whose k-steps hold a value in need of the full definition (bit k of `odd`): a rolled loop
-    // over the k-steps in which every step passes through the plain block (the skipping one if the tile holds zeros
+    // a full k-tile some of whose k-steps hold a value in need of the full definition (bit k of `odd`): a loop over
+    // pairs of k-steps in which every step passes through the plain block (the skipping one if the tile holds zeros
     // too, ZEROS) -- under an empty lane mask in the marked steps, whose products the full definition then adds.
+    // The fragments of the step after are read while a step is computed, in two sets of registers that the pair
+    // alternates (one step per round of the loop and no reading ahead spent 26 instructions around every block and
+    // most of the tile's time waiting for LDS).
     auto mixed_tile = [&](uint32_t odd, auto holds_zeros) __attribute__((always_inline)) {
         if constexpr (MODE != MODE_STD && TM == 4 && TN == 4) {
             constexpr bool ZEROS = decltype(holds_zeros)::value;
             typedef const __attribute__((address_space(3))) uint32_t* LdsWord;
             uint32_t pl = (uint32_t)(uintptr_t)(LdsWord)sl, pr = (uint32_t)(uintptr_t)(LdsWord)sr;
             const uint32_t to_plx = (uint32_t)(uintptr_t)(LdsWord)slx - pl, to_prx = (uint32_t)(uintptr_t)(LdsWord)srx - pr;
-#pragma unroll 1
-            for (int kk = 0; kk < BK; ++kk) {
-                if (BK == 32 && kk == 16) { pl += to_plx; pr += to_prx; }        // (see swizzled)
-                const u32x4 va = *reinterpret_cast<LdsVec>(pl), vb = *reinterpret_cast<LdsVec>(pr);
-                pl += LDL * 4; pr += LDR * 4;
+            auto step = [&](int kk, u32x4& va, u32x4& vb) __attribute__((always_inline)) {
                 // a marked step concerns the wavefronts whose lanes hold one of its odd values: 16 of a work-group's 256
                 // lanes for a value of the left operand, 16 per wavefront for one of the right operand
                 bool marked = ((odd >> kk) & 1u) != 0;
+                uint32_t half = ~0u;                   // the step's lane mask, wavefront-uniform: all lanes, or none (kept in scalar registers)
                 if (__builtin_expect(marked, 0)) {
                     constexpr uint32_t kUnstage = MODE == MODE_PAM ? kBias : 0u;      // the right operand is staged less the bias
-                    const bool mine = needs_full_definition(va.x) || needs_full_definition(va.y) || needs_full_definition(va.z)
-                                   || needs_full_definition(va.w) || needs_full_definition(vb.x + kUnstage) || needs_full_definition(vb.y + kUnstage)
-                                   || needs_full_definition(vb.z + kUnstage) || needs_full_definition(vb.w + kUnstage);
+                    const uint32_t ua[4] = {va.x, va.y, va.z, va.w}, ub[4] = {vb.x + kUnstage, vb.y + kUnstage, vb.z + kUnstage, vb.w + kUnstage};
+                    bool oa[4], ob[4], mine = false;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { oa[i] = needs_full_definition(ua[i]); ob[i] = needs_full_definition(ub[i]); mine |= oa[i] || ob[i]; }
                     marked = __ballot(mine) != 0ull;
+                    if constexpr (MODE == MODE_PAM) {
+                        // Tiny odd values (subnormal, or below 2^-63) mostly change nothing: |a (*) b| < 2^(Ea + Eb - 252)
+                        // for biased exponent fields Ea, Eb (a subnormal number's is 0; a PAM product is no larger than the
+                        // true one), and a sum whose field is at least Ea + Eb - 96 is left as it is by adding anything that
+                        // small (below an eighth of its last place).  Such a value is replaced by 2^-63, the smallest the
+                        // plain block takes: if every sum that one of its products goes to passes that test with 2^-63 in its
+                        // place -- which covers the value itself, it is smaller -- the step runs the plain block on the
+                        // replaced fragments and adds products that change nothing, as the true ones would.  Otherwise
+                        // (small sums, or an odd value that is inf, NaN or huge) the step takes the full definition.
+                        if (marked) {
+                            constexpr uint32_t kLeast = kPlainExpMin << 23;
+                            bool fits = true;
+#pragma unroll
+                            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const int ea = oa[i] ? (int)kPlainExpMin : (int)((ua[i] >> 23) & 0xffu);
+                                    const int eb = ob[j] ? (int)kPlainExpMin : (int)((ub[j] >> 23) & 0xffu);
+                                    const int es = (int)((f2u(acc[i][j]) >> 23) & 0xffu);
+                                    const bool tiny = (!oa[i] || ((ua[i] >> 23) & 0xffu) < kPlainExpMin) && (!ob[j] || ((ub[j] >> 23) & 0xffu) < kPlainExpMin);
+                                    fits &= !(oa[i] || ob[j]) || (tiny && es >= ea + eb - 96);
+                                }
+                            if (__ballot(!fits) == 0ull) {
+                                va.x = oa[0] ? kLeast : va.x; va.y = oa[1] ? kLeast : va.y; va.z = oa[2] ? kLeast : va.z; va.w = oa[3] ? kLeast : va.w;
+                                vb.x = ob[0] ? kLeast - kUnstage : vb.x; vb.y = ob[1] ? kLeast - kUnstage : vb.y;
+                                vb.z = ob[2] ? kLeast - kUnstage : vb.z; vb.w = ob[3] ? kLeast - kUnstage : vb.w;
+                                marked = false;
+                            }
+                        }
+                    }
+                    half = __builtin_amdgcn_readfirstlane(marked ? 0u : ~0u);
                 }
-                const uint32_t half = __builtin_amdgcn_readfirstlane(marked ? 0u : ~0u);     // (keeps the mask in scalar registers)
                 const uint64_t run = ((uint64_t)half << 32) | half;
                 if constexpr (MODE == MODE_PAM) {
                     if constexpr (ZEROS) pam_mac_4x4_skip_both_under(acc, va, vb, pl, pr, run);
@@ -1063,6 +1094,19 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                     const uint32_t a[4] = {va.x, va.y, va.z, va.w}, b[4] = {vb.x, vb.y, vb.z, vb.w};
                     guarded_products(a, b);
                 }
+            };
+            u32x4 fa0 = *reinterpret_cast<LdsVec>(pl), fb0 = *reinterpret_cast<LdsVec>(pr), fa1, fb1;
+#pragma unroll 1
+            for (int kk = 0; kk < BK; kk += 2) {
+                pl += LDL * 4; pr += LDR * 4;
+                fa1 = *reinterpret_cast<LdsVec>(pl); fb1 = *reinterpret_cast<LdsVec>(pr);
+                step(kk, fa0, fb0);
+                // (the last pair reads its own second step again: a read under a condition would make the wait before
+                // the block below one for all reads, the two just issued included)
+                pl += kk + 2 < BK ? LDL * 4 : 0; pr += kk + 2 < BK ? LDR * 4 : 0;
+                if (BK == 32 && kk == 14) { pl += to_plx; pr += to_prx; }        // (see swizzled)
+                fa0 = *reinterpret_cast<LdsVec>(pl); fb0 = *reinterpret_cast<LdsVec>(pr);
+                step(kk + 1, fa1, fb1);
             }
         }
     };

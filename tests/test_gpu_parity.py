@@ -301,6 +301,30 @@ def test_matmul_few_specials_per_k_tile(K, oracle):
                     assert_same_bits(host(K.pam_matmul_bwd(ta, tb, dev(D), True, True, delta_l, 1.0)), want, f"exact k={k} {la} x {lb}")
 
 
+def test_matmul_tiny_values_next_to_small_sums(K, oracle):
+    """A tiny value (subnormal, or below 2^-63) may pass as a zero in its k-step only where its products cannot change
+    the sums they go to.  Here the sums are small themselves (about 2^-57), the tiny values' exponents run from far below
+    to just below the plain range, and their products straddle the sums' last place: some k-steps take the full
+    definition, some skip, and every sum must still carry the bits of the plain ascending-k order."""
+    rng = np.random.RandomState(77)
+    for k, scale_b in ((256, 1.0), (96, 2.0 ** -20)):
+        A = (rng.standard_normal((150, k)) * 2.0 ** -60).astype(np.float32)
+        B = (rng.standard_normal((k, 90)) * scale_b).astype(np.float32)
+        flat = A.reshape(-1)
+        idx = rng.choice(flat.size, size=flat.size // 150, replace=False)
+        flat[idx] = (rng.uniform(1.0, 2.0, idx.size) * 2.0 ** rng.randint(-140, -63, idx.size) * rng.choice([-1.0, 1.0], idx.size)).astype(np.float32)
+        fb = B.reshape(-1)
+        jdx = rng.choice(fb.size, size=fb.size // 400, replace=False)
+        fb[jdx] = (rng.uniform(1.0, 2.0, jdx.size) * 2.0 ** rng.randint(-149, -63, jdx.size)).astype(np.float32)
+        want = ogemm(oracle, A, B)
+        assert np.isfinite(want).all() and np.count_nonzero(want) > want.size // 2
+        for la, ta in _layouts(A).items():
+            assert_same_bits(host(K.pam_matmul_fwd(ta, dev(B), True, True, 1.0)), want, f"k={k} {la}")
+        assert_same_bits(host(K.pam_matmul_fwd(dev(A), dev(B), True, True, 1.0552)), ogemm(oracle, A, B, offset=1.0552), f"k={k} offset")
+        # the same with the roles exchanged (tiny values mostly in the right operand)
+        assert_same_bits(host(K.pam_matmul_fwd(dev(B.T.copy()), dev(A.T.copy()), True, True, 1.0)), ogemm(oracle, B.T.copy(), A.T.copy()), f"k={k} exchanged")
+
+
 def test_bmm_tails_and_strides(K, oracle):
     # the reference's own bmm test shape (pam/test_pam.py:198-205): power-of-two weights => equals bmm
     rng = np.random.RandomState(6)
