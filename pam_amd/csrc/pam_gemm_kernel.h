@@ -1048,8 +1048,13 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                     constexpr uint32_t kUnstage = MODE == MODE_PAM ? kBias : 0u;      // the right operand is staged less the bias
                     const uint32_t ua[4] = {va.x, va.y, va.z, va.w}, ub[4] = {vb.x + kUnstage, vb.y + kUnstage, vb.z + kUnstage, vb.w + kUnstage};
                     bool oa[4], ob[4], mine = false;
+                    // (a tile without zeros tells its odd values by the staging's window test, two instructions a value)
+                    auto is_odd = [](uint32_t u) __attribute__((always_inline)) {
+                        if constexpr (ZEROS || MODE != MODE_PAM) return needs_full_definition(u);
+                        else return window(u) >= kWindowSpan;
+                    };
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) { oa[i] = needs_full_definition(ua[i]); ob[i] = needs_full_definition(ub[i]); mine |= oa[i] || ob[i]; }
+                    for (int i = 0; i < 4; ++i) { oa[i] = is_odd(ua[i]); ob[i] = is_odd(ub[i]); mine |= oa[i] || ob[i]; }
                     marked = __ballot(mine) != 0ull;
                     if constexpr (MODE == MODE_PAM) {
                         // Tiny odd values (subnormal, or below 2^-63) mostly change nothing: |a (*) b| < 2^(Ea + Eb - 252)
@@ -1062,16 +1067,27 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
                         // (small sums, or an odd value that is inf, NaN or huge) the step takes the full definition.
                         if (marked) {
                             constexpr uint32_t kLeast = kPlainExpMin << 23;
+                            // (row by row and column by column, and only those that hold an odd value somewhere in the
+                            // wavefront: mostly one of the eight)
                             bool fits = true;
+                            auto pair_fits = [&](int i, int j) __attribute__((always_inline)) {
+                                const uint32_t fa = (ua[i] >> 23) & 0xffu, fb = (ub[j] >> 23) & 0xffu;
+                                const int ea = oa[i] ? (int)kPlainExpMin : (int)fa, eb = ob[j] ? (int)kPlainExpMin : (int)fb;
+                                const int es = (int)((f2u(acc[i][j]) >> 23) & 0xffu);
+                                const bool tiny = (!oa[i] || fa < kPlainExpMin) && (!ob[j] || fb < kPlainExpMin);
+                                return tiny && es >= ea + eb - 96;
+                            };
 #pragma unroll
                             for (int i = 0; i < 4; ++i)
+                                if (__ballot(oa[i]) != 0ull) {
 #pragma unroll
-                                for (int j = 0; j < 4; ++j) {
-                                    const int ea = oa[i] ? (int)kPlainExpMin : (int)((ua[i] >> 23) & 0xffu);
-                                    const int eb = ob[j] ? (int)kPlainExpMin : (int)((ub[j] >> 23) & 0xffu);
-                                    const int es = (int)((f2u(acc[i][j]) >> 23) & 0xffu);
-                                    const bool tiny = (!oa[i] || ((ua[i] >> 23) & 0xffu) < kPlainExpMin) && (!ob[j] || ((ub[j] >> 23) & 0xffu) < kPlainExpMin);
-                                    fits &= !(oa[i] || ob[j]) || (tiny && es >= ea + eb - 96);
+                                    for (int j = 0; j < 4; ++j) fits &= !oa[i] || pair_fits(i, j);
+                                }
+#pragma unroll
+                            for (int j = 0; j < 4; ++j)
+                                if (__ballot(ob[j]) != 0ull) {
+#pragma unroll
+                                    for (int i = 0; i < 4; ++i) fits &= !ob[j] || pair_fits(i, j);
                                 }
                             if (__ballot(!fits) == 0ull) {
                                 va.x = oa[0] ? kLeast : va.x; va.y = oa[1] ? kLeast : va.y; va.z = oa[2] ? kLeast : va.z; va.w = oa[3] ? kLeast : va.w;
