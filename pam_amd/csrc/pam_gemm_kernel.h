@@ -784,21 +784,26 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
         // the shift-add and max per value below plus an integer add for the operand that carries the bias.
         constexpr bool kOffL = Stager<MODE, false>::kTakesOffset, kOffR = Stager<MODE, true>::kTakesOffset;
         const bool shifted = g.has_off == 1;
-        const uint32_t worst = max(ll.window_max(kOffL && shifted, g.off_add), rl.window_max(kOffR && shifted, g.off_add));
-        if (__builtin_expect(__ballot(worst >= kWindowSpan) == 0ull && g.has_off != 2, 1)) {
-            PlainStager<true> plus{(MODE == MODE_PAM ? 0u - kBias : 0u) + (shifted ? g.off_add : 0u)};
-            if (kOffL && (MODE == MODE_PAM || shifted)) ll.store(lds_l[buf], tid, plus); else ll.store(lds_l[buf], tid, same);
-            if (kOffR && (MODE == MODE_PAM || shifted)) rl.store(lds_r[buf], tid, plus); else rl.store(lds_r[buf], tid, same);
+        // (per operand: the zeros of a ReLU or of an image's padding sit in one of them, and the other one's values then
+        // need no look each)
+        const bool quick_l = __ballot(ll.window_max(kOffL && shifted, g.off_add) >= kWindowSpan) == 0ull && !(kOffL && g.has_off == 2);
+        const bool quick_r = __ballot(rl.window_max(kOffR && shifted, g.off_add) >= kWindowSpan) == 0ull && !(kOffR && g.has_off == 2);
+        PlainStager<true> plus{(MODE == MODE_PAM ? 0u - kBias : 0u) + (shifted ? g.off_add : 0u)};
+        if (quick_l) { if (kOffL && (MODE == MODE_PAM || shifted)) ll.store(lds_l[buf], tid, plus); else ll.store(lds_l[buf], tid, same); }
+        if (quick_r) { if (kOffR && (MODE == MODE_PAM || shifted)) rl.store(lds_r[buf], tid, plus); else rl.store(lds_r[buf], tid, same); }
+        if (__builtin_expect(quick_l && quick_r, 1)) {
             if (lane == 0) lds_flag[buf][wave] = 0u;      // (its k mask keeps an older value: readers go by the flag)
             return;
         }
         Stager<MODE, false> sl; Stager<MODE, true> sr;
-        if (has_off) {
-            if (Stager<MODE, false>::kTakesOffset) ll.apply_offset(g.off);
-            if (Stager<MODE, true>::kTakesOffset) rl.apply_offset(g.off);
+        if (!quick_l) {
+            if (has_off && Stager<MODE, false>::kTakesOffset) ll.apply_offset(g.off);
+            ll.store(lds_l[buf], tid, sl);
         }
-        ll.store(lds_l[buf], tid, sl);
-        rl.store(lds_r[buf], tid, sr);
+        if (!quick_r) {
+            if (has_off && Stager<MODE, true>::kTakesOffset) rl.apply_offset(g.off);
+            rl.store(lds_r[buf], tid, sr);
+        }
         const uint32_t found = (__ballot(sl.out_of_range() || sr.out_of_range()) != 0ull ? kGuarded : 0u)
                              | (__ballot(sl.zero) != 0ull ? kZerosL : 0u) | (__ballot(sr.zero) != 0ull ? kZerosR : 0u);
         if (lane == 0) lds_flag[buf][wave] = found;
