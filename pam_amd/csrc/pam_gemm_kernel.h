@@ -1033,10 +1033,10 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
     constexpr bool kSkips = MODE == MODE_PAM && TM == 4 && TN == 4;
 
     // a full k-tile some of whose k-steps hold a value in need of the full definition (bit k of `odd`): a loop over
-    // pairs of k-steps in which every step passes through the plain block (the skipping one if the tile holds zeros
+    // fours of k-steps in which every step passes through the plain block (the skipping one if the tile holds zeros
     // too, ZEROS) -- under an empty lane mask in the marked steps, whose products the full definition then adds.
-    // The fragments of the step after are read while a step is computed, in two sets of registers that the pair
-    // alternates (one step per round of the loop and no reading ahead spent 26 instructions around every block and
+    // The fragments of the step after are read while a step is computed, in two sets of registers that the steps
+    // alternate (one step per round of the loop and no reading ahead spent 26 instructions around every block and
     // most of the tile's time waiting for LDS).
     auto mixed_tile = [&](uint32_t odd, auto holds_zeros) __attribute__((always_inline)) {
         if constexpr (MODE != MODE_STD && TM == 4 && TN == 4) {
@@ -1118,16 +1118,22 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             };
             u32x4 fa0 = *reinterpret_cast<LdsVec>(pl), fb0 = *reinterpret_cast<LdsVec>(pr), fa1, fb1;
 #pragma unroll 1
-            for (int kk = 0; kk < BK; kk += 2) {
+            for (int kk = 0; kk < BK; kk += 4) {
                 pl += LDL * 4; pr += LDR * 4;
                 fa1 = *reinterpret_cast<LdsVec>(pl); fb1 = *reinterpret_cast<LdsVec>(pr);
                 step(kk, fa0, fb0);
-                // (the last pair reads its own second step again: a read under a condition would make the wait before
-                // the block below one for all reads, the two just issued included)
-                pl += kk + 2 < BK ? LDL * 4 : 0; pr += kk + 2 < BK ? LDR * 4 : 0;
-                if (BK == 32 && kk == 14) { pl += to_plx; pr += to_prx; }        // (see swizzled)
+                pl += LDL * 4; pr += LDR * 4;
                 fa0 = *reinterpret_cast<LdsVec>(pl); fb0 = *reinterpret_cast<LdsVec>(pr);
                 step(kk + 1, fa1, fb1);
+                pl += LDL * 4; pr += LDR * 4;
+                fa1 = *reinterpret_cast<LdsVec>(pl); fb1 = *reinterpret_cast<LdsVec>(pr);
+                step(kk + 2, fa0, fb0);
+                // (the last four read their own last step again: a read under a condition would make the wait before
+                // the block below one for all reads, the two just issued included)
+                pl += kk + 4 < BK ? LDL * 4 : 0; pr += kk + 4 < BK ? LDR * 4 : 0;
+                if (BK == 32 && kk == 12) { pl += to_plx; pr += to_prx; }        // (see swizzled)
+                fa0 = *reinterpret_cast<LdsVec>(pl); fb0 = *reinterpret_cast<LdsVec>(pr);
+                step(kk + 3, fa1, fb1);
             }
         }
     };
