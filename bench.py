@@ -304,6 +304,16 @@ def main():
         # one value in a thousand of the left operand a subnormal number: its k-step takes the full definition, the rest of its k-tile not
         X2n = torch.where((torch.rand(X2.shape, generator=g) < 1e-3).to(dev), torch.full_like(X2, 1e-40), X2)
         exact["fwd_12608x192x768_0.1pct_subnormal_input"] = (2, macs_each, lambda: K.pam_matmul_fwd(X2n, W2.T, True, False, 1.0))
+        # the other linear layers of the same model (qkv 192->576, proj 192->192) and the MLP block at the DeiT-small
+        # and DeiT-base widths, same 12608 tokens: forward, dX, dW
+        for d_in, d_out in ((192, 576), (192, 192), (384, 1536), (768, 3072)):
+            Xw = torch.randn(T, d_in, generator=g).to(dev)
+            Ww = torch.nn.init.trunc_normal_(torch.empty(d_out, d_in), std=0.02, a=-0.04, b=0.04, generator=g).to(dev)
+            dYw = (torch.randn(T, d_out, generator=g) * 1e-2).to(dev)
+            mm = T * d_in * d_out
+            exact[f"fwd_12608x{d_out}x{d_in}"] = (2, mm, lambda Xw=Xw, Ww=Ww: K.pam_matmul_fwd(Xw, Ww.T, True, False, 1.0))
+            exact[f"dX_12608x{d_in}x{d_out}"] = (2, mm, lambda dYw=dYw, Ww=Ww: K.pam_matmul_fwd(dYw, Ww, True, True, 1.0))
+            exact[f"dW_{d_in}x{d_out}x12608"] = (2, mm, lambda Xw=Xw, dYw=dYw: K.pam_matmul_fwd(Xw.T, dYw, False, True, 1.0))
         for name, (ops, macs, fn) in exact.items():
             ms = event_time_ms(fn, 30, torch)
             other[name] = {"ms": round(ms, 4), "gmacs": round(macs / ms / 1e6, 1), "valu_frac": round(ops * macs / (ms * 1e-3) / lane_peak, 4)}
