@@ -315,29 +315,56 @@ __device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, 
     p = p - pam_mul_off(pad_div_off(m, denom, off, ho), a.step_size, off, ho);
 }
 
-__global__ __launch_bounds__(kThreads) void adam_vec_kernel(v4f* __restrict__ p, const v4f* __restrict__ g,
-                                                           v4f* __restrict__ m, v4f* __restrict__ v, size_t nvec, AdamArgs a)
+// kAdamVectors 128-bit vectors per lane and stream, all loads issued before the arithmetic, everything read and
+// written past the caches (each value is touched once per step): 345 -> 315 us for 2^26 parameters against one vector
+// per lane with cached loads.
+__device__ __forceinline__ void adam_vector(v4f& pp, const v4f& gg, v4f& mm, v4f& vv, const AdamArgs& a)
 {
-    const size_t step = (size_t)gridDim.x * kThreads;
-    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += step) {
-        v4f pp = p[i], gg = __builtin_nontemporal_load(g + i), mm = m[i], vv = v[i];
-        v4f p1 = pp, m1 = mm, v1 = vv;
-        Span sp;
+    v4f p1 = pp, m1 = mm, v1 = vv;
+    Span sp;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        float pc = pp[c], mc = mm[c], vc = vv[c];
+        adam_one_unchecked(pc, gg[c], mc, vc, a, sp);
+        p1[c] = pc; m1[c] = mc; v1[c] = vc;
+    }
+    if (!sp.normal()) {                     // a zero, subnormal, inf, NaN or out-of-range value somewhere: redo checked
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             float pc = pp[c], mc = mm[c], vc = vv[c];
-            adam_one_unchecked(pc, gg[c], mc, vc, a, sp);
+            adam_one(pc, gg[c], mc, vc, a);
             p1[c] = pc; m1[c] = mc; v1[c] = vc;
         }
-        if (!sp.normal()) {                     // a zero, subnormal, inf, NaN or out-of-range value somewhere: redo checked
+    }
+    pp = p1; mm = m1; vv = v1;
+}
+
+constexpr int kAdamVectors = 2;               // 128-bit vectors per lane and stream (four measured the same)
+__global__ __launch_bounds__(kThreads) void adam_vec_kernel(v4f* __restrict__ p, const v4f* __restrict__ g,
+                                                           v4f* __restrict__ m, v4f* __restrict__ v, size_t nvec, AdamArgs a)
+{
+    // work-group b takes kAdamVectors x kThreads consecutive vectors: lane t the vectors t, t + kThreads, ... of them
+    const size_t first = (size_t)blockIdx.x * (kAdamVectors * kThreads) + threadIdx.x;
+    if (first + (kAdamVectors - 1) * kThreads < nvec) {
+        v4f pp[kAdamVectors], gg[kAdamVectors], mm[kAdamVectors], vv[kAdamVectors];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                float pc = pp[c], mc = mm[c], vc = vv[c];
-                adam_one(pc, gg[c], mc, vc, a);
-                p1[c] = pc; m1[c] = mc; v1[c] = vc;
-            }
+        for (int u = 0; u < kAdamVectors; ++u) {
+            const size_t i = first + (size_t)u * kThreads;
+            pp[u] = __builtin_nontemporal_load(p + i); gg[u] = __builtin_nontemporal_load(g + i);
+            mm[u] = __builtin_nontemporal_load(m + i); vv[u] = __builtin_nontemporal_load(v + i);
         }
-        p[i] = p1; m[i] = m1; v[i] = v1;
+#pragma unroll
+        for (int u = 0; u < kAdamVectors; ++u) {
+            const size_t i = first + (size_t)u * kThreads;
+            adam_vector(pp[u], gg[u], mm[u], vv[u], a);
+            __builtin_nontemporal_store(pp[u], p + i); __builtin_nontemporal_store(mm[u], m + i); __builtin_nontemporal_store(vv[u], v + i);
+        }
+    } else {
+        for (size_t i = first; i < nvec; i += kThreads) {
+            v4f p0 = p[i], g0 = g[i], m0 = m[i], v0 = v[i];
+            adam_vector(p0, g0, m0, v0, a);
+            p[i] = p0; m[i] = m0; v[i] = v0;
+        }
     }
 }
 
@@ -448,8 +475,8 @@ int pam_hip_adam_step(float* p, const float* g, float* m, float* v, size_t n, fl
     size_t nvec = (align & 15u) ? 0 : n / 4;
     const size_t cap = (size_t)1 << 30;
     if (nvec) {
-        size_t blocks = (nvec + kThreads - 1) / kThreads;
-        if (blocks > cap) blocks = cap;
+        const size_t blocks = (nvec + kAdamVectors * kThreads - 1) / (kAdamVectors * kThreads);
+        if (blocks > cap) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "adam_step: more than 2^41 parameters");
         hipLaunchKernelGGL(adam_vec_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, st, (v4f*)p, (const v4f*)g, (v4f*)m,
                            (v4f*)v, nvec, a);
     }
