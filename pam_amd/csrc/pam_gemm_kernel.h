@@ -65,7 +65,7 @@ namespace pamgemm {
 using namespace pamdev;
 
 enum { MODE_PAM = 0, MODE_STD = 1, MODE_BWD_DL = 2, MODE_BWD_DR = 3 };
-enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3 };   // k contiguous / row contiguous / any strides / image patches
+enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3, LOAD_CONVQ = 4 };   // k contiguous / row contiguous / any strides / image patches / ... in 128-bit quads
 
 constexpr int KGRAN = 32;         // k ranges handed to work-groups are multiples of this
 constexpr int PAD = 4;
@@ -81,7 +81,10 @@ struct Operand { const float* p; long sb, sr, sk; };    // batch, row (the non-k
 // and per l, the address part and the coordinates: {c H W + di W + dj, di << 16 | dj} and
 // {h0 W + w0, h0 << 16 | (w0 & 0xffff)}.  `transposed` exchanges the roles of the operand's two
 // indices (the matrix is then [Ho Wo, C kh kw]: the weight-gradient product).
-struct ConvGeom { const int2* ktab; const int2* ltab; int H, W; int transposed; };
+// `quads`: no padding, and the kernel's width, the image's width and the horizontal stride are multiples of four (the
+// patch embeddings of vision transformers: 16 x 16 patches at stride 16): four consecutive k of one patch are then four
+// consecutive, 16-byte aligned values of an image row and always inside the image, and the loader fetches them as one.
+struct ConvGeom { const int2* ktab; const int2* ltab; int H, W; int transposed; int quads; };
 
 struct GemmArgs {
     Operand L, R;
@@ -175,8 +178,10 @@ struct TileLoader {
     static constexpr int kVecs = ROWS * BK / 4 / NT;      // float4 per lane (vector kinds)
     static constexpr int kElems = ROWS * BK / NT;         // scalars per lane (generic kind)
     static_assert(ROWS * BK % (4 * NT) == 0 && NT % ROWS == 0, "tile must divide over the work-group");
+    static constexpr bool kKQuads = KIND == LOAD_KVEC || KIND == LOAD_CONVQ;      // 128-bit loads along k
     float4 v[kVecs > 0 ? kVecs : 1];
     int2 fixed; bool have_fixed = false;          // LOAD_CONV: the lane's own table entry
+    int patch_at[kVecs > 0 ? kVecs : 1];          // LOAD_CONVQ: where the patches of the lane's rows begin in the image
 
     __device__ __forceinline__ void load(const Operand& op, const float* base, int row0, int nrows, int k0, int kend, int tid,
                                          const ConvGeom& cv)
@@ -203,6 +208,20 @@ struct TileLoader {
                 const int h = (le.y >> 16) + (ke.y >> 16), w = (int)(short)(le.y & 0xffff) + (ke.y & 0xffff);
                 const bool inside = (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
                 s[i] = inside ? base[ke.x + le.x] : 0.0f;
+            }
+        } else if (KIND == LOAD_CONVQ) {
+            // as LOAD_KVEC, the address from the two tables: the rows' entries once per work-group, k's per k-tile
+            typedef const __attribute__((address_space(4))) int* ConstTable;
+            if (!have_fixed) {
+#pragma unroll
+                for (int i = 0; i < kVecs; ++i) patch_at[i] = cv.ltab[min(row0 + (tid + i * NT) / (BK / 4), nrows - 1)].x;
+                have_fixed = true;
+            }
+            ConstTable ktab = (ConstTable)cv.ktab;
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                const int k = min(k0 + ((tid + i * NT) % (BK / 4)) * 4, kend - 4);
+                v[i] = *reinterpret_cast<const float4*>(base + patch_at[i] + ktab[2 * k]);
             }
         } else if (KIND == LOAD_KVEC) {
 #pragma unroll
@@ -239,7 +258,7 @@ struct TileLoader {
     // (an operand that takes a normal offset must be in range before and after it)
     __device__ __forceinline__ uint32_t window_max(bool shifted, uint32_t add) const
     {
-        constexpr int n = (KIND == LOAD_KVEC || KIND == LOAD_RVEC) ? 4 * kVecs : kElems;
+        constexpr int n = (kKQuads || KIND == LOAD_RVEC) ? 4 * kVecs : kElems;
         const float* s = reinterpret_cast<const float*>(v);
         uint32_t m = 0;
 #pragma unroll
@@ -269,7 +288,7 @@ struct TileLoader {
     __device__ __forceinline__ void odd_by_k(int tid, uint32_t& odd) const
     {
         auto see = [&](float f, int k) __attribute__((always_inline)) { odd |= (uint32_t)needs_full_definition(f2u(f)) << k; };
-        if (KIND == LOAD_KVEC) {
+        if (kKQuads) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 const int k = ((tid + i * NT) % (BK / 4)) * 4;
@@ -292,7 +311,7 @@ struct TileLoader {
     __device__ __forceinline__ void store(uint32_t* lds, int tid, S& st)
     {
         constexpr int LD = ROWS + PAD;
-        if (KIND == LOAD_KVEC) {
+        if (kKQuads) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 int id = tid + i * NT;
@@ -1271,6 +1290,7 @@ void launch_gemm(int lk, int rk, unsigned groups, hipStream_t st, const GemmArgs
     PAM_GEMM_CASE(LOAD_ANY, LOAD_KVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_RVEC) PAM_GEMM_CASE(LOAD_ANY, LOAD_ANY)
     if constexpr (MODE != MODE_STD) {                                  // image patches as the right operand
         PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_RVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_ANY, LOAD_CONV)
+        if constexpr (MODE == MODE_PAM) { PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONVQ) }      // (forward products of patch embeddings)
     }
 #undef PAM_GEMM_CASE
 }

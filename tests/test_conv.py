@@ -16,7 +16,9 @@ CASES = [
     # batch, c, h, w, co, kh, kw, stride, padding
     (2, 3, 9, 8, 5, 3, 3, (1, 1), (1, 1)),
     (3, 6, 12, 10, 70, 3, 5, (2, 1), (0, 2)),
-    (2, 4, 16, 16, 8, 4, 4, (4, 4), (0, 0)),          # non-overlapping patches (patch embedding)
+    (2, 4, 16, 16, 8, 4, 4, (4, 4), (0, 0)),          # non-overlapping patches (patch embedding): 128-bit patch loads
+    (2, 3, 32, 40, 70, 8, 8, (8, 8), (0, 0)),         # ... with k = 192 (32-deep k-tiles), ragged in both outputs
+    (1, 2, 20, 24, 5, 8, 8, (4, 4), (0, 0)),          # ... overlapping patches, k = 128
     (1, 20, 7, 7, 33, 1, 1, (1, 1), (0, 0)),
     (2, 16, 32, 32, 64, 3, 3, (1, 1), (1, 1)),
 ]
