@@ -245,12 +245,14 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
         g.off_add = bits - kBias;
     }
 
-    g.cv = conv ? *conv : ConvGeom{nullptr, nullptr, 0, 0, 0, 0};
+    g.cv = conv ? *conv : ConvGeom{nullptr, nullptr, 0, 0, 0, 0, 0};
 
     int lk = load_kind(l_sr, l_sc, l_sb, l, M, K);
     int rk = conv ? LOAD_CONV : load_kind(r_sc, r_sr, r_sb, r, N, K);
     if (conv && conv->quads && !conv->transposed && mode == MODE_PAM && lk == LOAD_KVEC && K % 4 == 0 && (reinterpret_cast<uintptr_t>(r) & 15u) == 0 && r_sb % 4 == 0)
         rk = LOAD_CONVQ;
+    else if (conv && conv->row_quads && !conv->transposed && mode != MODE_STD && lk == LOAD_KVEC && N % 4 == 0)
+        rk = LOAD_CONVR;
     switch (mode) {
     case MODE_PAM: launch_mode<MODE_PAM>(p, lk, rk, st, g); break;
     case MODE_STD: launch_mode<MODE_STD>(p, lk, rk, st, g); break;
@@ -344,7 +346,8 @@ int conv_prepare(const char* what, const ConvShape& s, const ConvSpace& sp, void
     hipLaunchKernelGGL(conv_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, ktab, ltab, (int)s.K(), (int)s.L(),
                        (int)s.kh, (int)s.kw, (int)s.h, (int)s.w, (int)s.wo, (int)s.sh, (int)s.sw, (int)s.ph, (int)s.pw);
     const bool quads = s.ph == 0 && s.pw == 0 && s.kw % 4 == 0 && s.w % 4 == 0 && s.sw % 4 == 0;
-    cv = ConvGeom{ktab, ltab, (int)s.h, (int)s.w, transposed ? 1 : 0, quads ? 1 : 0};
+    const bool row_quads = s.sw == 1 && s.wo % 4 == 0;
+    cv = ConvGeom{ktab, ltab, (int)s.h, (int)s.w, transposed ? 1 : 0, quads ? 1 : 0, row_quads ? 1 : 0};
     return PAM_HIP_OK;
 }
 

@@ -65,7 +65,7 @@ namespace pamgemm {
 using namespace pamdev;
 
 enum { MODE_PAM = 0, MODE_STD = 1, MODE_BWD_DL = 2, MODE_BWD_DR = 3 };
-enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3, LOAD_CONVQ = 4 };   // k contiguous / row contiguous / any strides / image patches / ... in 128-bit quads
+enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3, LOAD_CONVQ = 4, LOAD_CONVR = 5 };   // k contiguous / row contiguous / any strides / image patches / ... in quads along k / ... in quads of output positions
 
 constexpr int KGRAN = 32;         // k ranges handed to work-groups are multiples of this
 constexpr int PAD = 4;
@@ -84,7 +84,11 @@ struct Operand { const float* p; long sb, sr, sk; };    // batch, row (the non-k
 // `quads`: no padding, and the kernel's width, the image's width and the horizontal stride are multiples of four (the
 // patch embeddings of vision transformers: 16 x 16 patches at stride 16): four consecutive k of one patch are then four
 // consecutive, 16-byte aligned values of an image row and always inside the image, and the loader fetches them as one.
-struct ConvGeom { const int2* ktab; const int2* ltab; int H, W; int transposed; int quads; };
+// `row_quads`: horizontal stride 1 and an output width that is a multiple of four: four consecutive output positions are
+// then four consecutive pixels of one image row under every k, and the loader works out one address and one row test per
+// four values and hands the staging 128-bit vectors along the positions (padding allowed: the ends of a row are tested
+// per value).
+struct ConvGeom { const int2* ktab; const int2* ltab; int H, W; int transposed; int quads; int row_quads; };
 
 struct GemmArgs {
     Operand L, R;
@@ -179,6 +183,7 @@ struct TileLoader {
     static constexpr int kElems = ROWS * BK / NT;         // scalars per lane (generic kind)
     static_assert(ROWS * BK % (4 * NT) == 0 && NT % ROWS == 0, "tile must divide over the work-group");
     static constexpr bool kKQuads = KIND == LOAD_KVEC || KIND == LOAD_CONVQ;      // 128-bit loads along k
+    static constexpr bool kRQuads = KIND == LOAD_RVEC || KIND == LOAD_CONVR;      // ... along the rows
     float4 v[kVecs > 0 ? kVecs : 1];
     int2 fixed; bool have_fixed = false;          // LOAD_CONV: the lane's own table entry
     int patch_at[kVecs > 0 ? kVecs : 1];          // LOAD_CONVQ: where the patches of the lane's rows begin in the image
@@ -208,6 +213,25 @@ struct TileLoader {
                 const int h = (le.y >> 16) + (ke.y >> 16), w = (int)(short)(le.y & 0xffff) + (ke.y & 0xffff);
                 const bool inside = (unsigned)h < (unsigned)cv.H && (unsigned)w < (unsigned)cv.W;
                 s[i] = inside ? base[ke.x + le.x] : 0.0f;
+            }
+        } else if (KIND == LOAD_CONVR) {
+            // as LOAD_RVEC: vector i holds rows rq * 4 ... + 3 (four output positions of one image row) under one k
+            if (!have_fixed) {
+                fixed = cv.ltab[min(row0 + (tid % (ROWS / 4)) * 4, nrows - 4)];          // (the same rows for every vector of the lane)
+                have_fixed = true;
+            }
+            static_assert(NT % (ROWS / 4) == 0, "a lane's vectors must share their rows");
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                const int kk = min(k0 + (tid + i * NT) / (ROWS / 4), kend - 1);
+                const int2 ke = cv.ktab[kk];
+                const int h = (fixed.y >> 16) + (ke.y >> 16), w = (int)(short)(fixed.y & 0xffff) + (ke.y & 0xffff);
+                const bool row_inside = (unsigned)h < (unsigned)cv.H;
+                const float* at = base + (ke.x + fixed.x);
+                v[i].x = row_inside && (unsigned)w < (unsigned)cv.W ? at[0] : 0.0f;
+                v[i].y = row_inside && (unsigned)(w + 1) < (unsigned)cv.W ? at[1] : 0.0f;
+                v[i].z = row_inside && (unsigned)(w + 2) < (unsigned)cv.W ? at[2] : 0.0f;
+                v[i].w = row_inside && (unsigned)(w + 3) < (unsigned)cv.W ? at[3] : 0.0f;
             }
         } else if (KIND == LOAD_CONVQ) {
             // as LOAD_KVEC, the address from the two tables: the rows' entries once per work-group, k's per k-tile
@@ -258,7 +282,7 @@ struct TileLoader {
     // (an operand that takes a normal offset must be in range before and after it)
     __device__ __forceinline__ uint32_t window_max(bool shifted, uint32_t add) const
     {
-        constexpr int n = (kKQuads || KIND == LOAD_RVEC) ? 4 * kVecs : kElems;
+        constexpr int n = (kKQuads || kRQuads) ? 4 * kVecs : kElems;
         const float* s = reinterpret_cast<const float*>(v);
         uint32_t m = 0;
 #pragma unroll
@@ -294,7 +318,7 @@ struct TileLoader {
                 const int k = ((tid + i * NT) % (BK / 4)) * 4;
                 see(v[i].x, k); see(v[i].y, k + 1); see(v[i].z, k + 2); see(v[i].w, k + 3);
             }
-        } else if (KIND == LOAD_RVEC) {
+        } else if (kRQuads) {
 #pragma unroll
             for (int i = 0; i < kVecs; ++i) {
                 const int k = (tid + i * NT) / (ROWS / 4);
@@ -319,7 +343,7 @@ struct TileLoader {
                 d[0 * LD] = st.one(v[i].x); d[1 * LD] = st.one(v[i].y);
                 d[2 * LD] = st.one(v[i].z); d[3 * LD] = st.one(v[i].w);
             }
-        } else if (KIND == LOAD_RVEC) {
+        } else if (kRQuads) {
             // (vector i of a lane sits under k = i * kPer + tid / (ROWS / 4), the second term below kPer: which half of a
             // 32-deep tile that is depends on i alone, so the exchange of the row groups costs nothing per vector)
             constexpr int kPer = NT / (ROWS / 4);
@@ -1291,6 +1315,7 @@ void launch_gemm(int lk, int rk, unsigned groups, hipStream_t st, const GemmArgs
     if constexpr (MODE != MODE_STD) {                                  // image patches as the right operand
         PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_RVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_ANY, LOAD_CONV)
         if constexpr (MODE == MODE_PAM) { PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONVQ) }      // (forward products of patch embeddings)
+        PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONVR)                                          // (convolutions of horizontal stride 1)
     }
 #undef PAM_GEMM_CASE
 }
