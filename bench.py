@@ -351,14 +351,18 @@ def main():
             cm = cb * co_ * ho * ho * cc * ck * ck
             ms = event_time_ms(lambda: abi.conv2d_fwd(xc, wc, (cs, cs), (cp, cp), 1.0), 30, torch)
             other[tag] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1), "valu_frac": round(2 * cm / (ms * 1e-3) / lane_peak, 4)}
+            # the per-image weight gradients (the same patches, transposed), approximate and exact
+            gy = (torch.randn(cb, co_, ho, ho, generator=g) * 1e-2).to(dev)
+            for kind, exact_, ops in (("approx", False, 2), ("exact", True, 3)):
+                ms = event_time_ms(lambda: abi.conv2d_bwd_weight(xc, gy, wc, (cs, cs), (cp, cp), exact_, 1.0), 30, torch)
+                other[f"{tag}_weight_gradient_{kind}"] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1),
+                                                         "valu_frac": round(ops * cm / (ms * 1e-3) / lane_peak, 4)}
             if cs == 1:                 # the gradient of the input, also in place (a convolution of the upstream gradient)
-                gy = (torch.randn(cb, co_, ho, ho, generator=g) * 1e-2).to(dev)
                 for kind, exact_, ops in (("approx", False, 2), ("exact", True, 3)):
                     ms = event_time_ms(lambda: abi.conv2d_bwd_input(gy, wc, xc, (cp, cp), exact_, 1.0), 30, torch)
                     other[f"{tag}_input_gradient_{kind}"] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1),
                                                             "valu_frac": round(ops * cm / (ms * 1e-3) / lane_peak, 4)}
-                del gy
-            del xc, wc
+            del gy, xc, wc
         na = 1 << 26
         pa, ga, ma, va = (torch.randn(na, generator=g).to(dev) * s_ for s_ in (1.0, 1e-2, 1e-2, 1e-4))
         va.abs_()

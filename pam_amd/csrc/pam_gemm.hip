@@ -253,6 +253,8 @@ int gemm(const char* what, int mode, long batch, long M, long N, long K,
         rk = LOAD_CONVQ;
     else if (conv && conv->row_quads && !conv->transposed && mode != MODE_STD && lk == LOAD_KVEC && N % 4 == 0)
         rk = LOAD_CONVR;
+    else if (conv && conv->row_quads && conv->transposed && mode != MODE_STD && lk == LOAD_KVEC && K % 4 == 0)
+        rk = LOAD_CONVK;
     switch (mode) {
     case MODE_PAM: launch_mode<MODE_PAM>(p, lk, rk, st, g); break;
     case MODE_STD: launch_mode<MODE_STD>(p, lk, rk, st, g); break;

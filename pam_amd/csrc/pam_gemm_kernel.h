@@ -65,7 +65,7 @@ namespace pamgemm {
 using namespace pamdev;
 
 enum { MODE_PAM = 0, MODE_STD = 1, MODE_BWD_DL = 2, MODE_BWD_DR = 3 };
-enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3, LOAD_CONVQ = 4, LOAD_CONVR = 5 };   // k contiguous / row contiguous / any strides / image patches / ... in quads along k / ... in quads of output positions
+enum { LOAD_KVEC = 0, LOAD_RVEC = 1, LOAD_ANY = 2, LOAD_CONV = 3, LOAD_CONVQ = 4, LOAD_CONVR = 5, LOAD_CONVK = 6 };   // k contiguous / row contiguous / any strides / image patches / ... in quads along k / ... in quads of output positions / the same, transposed
 
 constexpr int KGRAN = 32;         // k ranges handed to work-groups are multiples of this
 constexpr int PAD = 4;
@@ -182,11 +182,12 @@ struct TileLoader {
     static constexpr int kVecs = ROWS * BK / 4 / NT;      // float4 per lane (vector kinds)
     static constexpr int kElems = ROWS * BK / NT;         // scalars per lane (generic kind)
     static_assert(ROWS * BK % (4 * NT) == 0 && NT % ROWS == 0, "tile must divide over the work-group");
-    static constexpr bool kKQuads = KIND == LOAD_KVEC || KIND == LOAD_CONVQ;      // 128-bit loads along k
+    static constexpr bool kKQuads = KIND == LOAD_KVEC || KIND == LOAD_CONVQ || KIND == LOAD_CONVK;      // 128-bit loads along k
     static constexpr bool kRQuads = KIND == LOAD_RVEC || KIND == LOAD_CONVR;      // ... along the rows
     float4 v[kVecs > 0 ? kVecs : 1];
     int2 fixed; bool have_fixed = false;          // LOAD_CONV: the lane's own table entry
     int patch_at[kVecs > 0 ? kVecs : 1];          // LOAD_CONVQ: where the patches of the lane's rows begin in the image
+    int2 row_entry[KIND == LOAD_CONVK && kVecs > 0 ? kVecs : 1];      // LOAD_CONVK: the k table's entries of the lane's rows
 
     __device__ __forceinline__ void load(const Operand& op, const float* base, int row0, int nrows, int k0, int kend, int tid,
                                          const ConvGeom& cv)
@@ -228,6 +229,25 @@ struct TileLoader {
                 const int h = (fixed.y >> 16) + (ke.y >> 16), w = (int)(short)(fixed.y & 0xffff) + (ke.y & 0xffff);
                 const bool row_inside = (unsigned)h < (unsigned)cv.H;
                 const float* at = base + (ke.x + fixed.x);
+                v[i].x = row_inside && (unsigned)w < (unsigned)cv.W ? at[0] : 0.0f;
+                v[i].y = row_inside && (unsigned)(w + 1) < (unsigned)cv.W ? at[1] : 0.0f;
+                v[i].z = row_inside && (unsigned)(w + 2) < (unsigned)cv.W ? at[2] : 0.0f;
+                v[i].w = row_inside && (unsigned)(w + 3) < (unsigned)cv.W ? at[3] : 0.0f;
+            }
+        } else if (KIND == LOAD_CONVK) {
+            // the transposed patches of a `row_quads` convolution (its weight gradient): the rows are (c, i, j) and k runs
+            // over the output positions, four consecutive ones per vector as in LOAD_CONVR, staged as LOAD_KVEC is
+            if (!have_fixed) {
+#pragma unroll
+                for (int i = 0; i < kVecs; ++i) row_entry[i] = cv.ktab[min(row0 + (tid + i * NT) / (BK / 4), nrows - 1)];
+                have_fixed = true;
+            }
+#pragma unroll
+            for (int i = 0; i < kVecs; ++i) {
+                const int2 le = cv.ltab[min(k0 + ((tid + i * NT) % (BK / 4)) * 4, kend - 4)], ke = row_entry[i];
+                const int h = (le.y >> 16) + (ke.y >> 16), w = (int)(short)(le.y & 0xffff) + (ke.y & 0xffff);
+                const bool row_inside = (unsigned)h < (unsigned)cv.H;
+                const float* at = base + (ke.x + le.x);
                 v[i].x = row_inside && (unsigned)w < (unsigned)cv.W ? at[0] : 0.0f;
                 v[i].y = row_inside && (unsigned)(w + 1) < (unsigned)cv.W ? at[1] : 0.0f;
                 v[i].z = row_inside && (unsigned)(w + 2) < (unsigned)cv.W ? at[2] : 0.0f;
@@ -1316,6 +1336,7 @@ void launch_gemm(int lk, int rk, unsigned groups, hipStream_t st, const GemmArgs
         PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_RVEC, LOAD_CONV) PAM_GEMM_CASE(LOAD_ANY, LOAD_CONV)
         if constexpr (MODE == MODE_PAM) { PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONVQ) }      // (forward products of patch embeddings)
         PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONVR)                                          // (convolutions of horizontal stride 1)
+        PAM_GEMM_CASE(LOAD_KVEC, LOAD_CONVK)                                          // (... their weight gradients)
     }
 #undef PAM_GEMM_CASE
 }

@@ -23,6 +23,7 @@ CASES = [
     (2, 16, 32, 32, 64, 3, 3, (1, 1), (1, 1)),          # horizontal stride 1, output width a multiple of 4: position quads
     (2, 32, 12, 16, 40, 3, 3, (1, 1), (1, 1)),          # ... with k = 288 (32-deep k-tiles)
     (1, 8, 11, 12, 9, 3, 5, (2, 1), (1, 2)),            # ... vertical stride 2, padding 2 at the row ends
+    (1, 4, 16, 32, 6, 3, 3, (1, 1), (1, 1)),            # ... 512 output positions (32-deep k-tiles in the weight gradient)
 ]
 
 
