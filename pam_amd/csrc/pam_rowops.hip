@@ -47,11 +47,28 @@ constexpr float kLn2 = (float)0.6931471805599453;        // math.log(2.0) rounde
 
 struct Offset { float off; bool has; };
 
+// The butterfly over a wavefront, lanes 32, 16, 8, 4, 2, 1 apart in that order, without a trip through LDS per step:
+// the two halves and then the rows of 16 lanes are exchanged by the swap instructions, and within a row lane l takes
+// the value 8, 4, 2, 1 lanes around the row from it (a DPP operand of the add).  After the step at distance 2d the
+// values repeat every 2d lanes, so the lane d around the row holds what the lane d apart (l ^ d) holds, and every lane
+// ends with the same bits as with exchanges between l and l ^ d.
+template <class F>
+__device__ __forceinline__ float wave_fold(float p, F f)
+{
+    typedef uint32_t Pair2 __attribute__((ext_vector_type(2)));
+    Pair2 r = __builtin_amdgcn_permlane32_swap(f2u(p), f2u(p), false, false);
+    p = f(u2f(r[0]), u2f(r[1]));
+    r = __builtin_amdgcn_permlane16_swap(f2u(p), f2u(p), false, false);
+    p = f(u2f(r[0]), u2f(r[1]));
+    p = f(p, u2f(__builtin_amdgcn_update_dpp(0u, f2u(p), 0x128, 0xf, 0xf, false)));       // row_ror:8
+    p = f(p, u2f(__builtin_amdgcn_update_dpp(0u, f2u(p), 0x124, 0xf, 0xf, false)));       // row_ror:4
+    p = f(p, u2f(__builtin_amdgcn_update_dpp(0u, f2u(p), 0x122, 0xf, 0xf, false)));       // row_ror:2
+    p = f(p, u2f(__builtin_amdgcn_update_dpp(0u, f2u(p), 0x121, 0xf, 0xf, false)));       // row_ror:1
+    return p;
+}
 __device__ __forceinline__ float wave_sum(float p)
 {
-#pragma unroll
-    for (int s = 32; s >= 1; s >>= 1) p = p + __shfl_xor(p, s, 64);
-    return p;
+    return wave_fold(p, [](float a, float b) { return a + b; });
 }
 
 // Who holds which element of a row and how partial sums over the row are combined.
@@ -94,8 +111,7 @@ struct MaxNan {
     __device__ __forceinline__ void take(float v) { if (v != v) nan = true; else mx = fmaxf(mx, v); }
     __device__ __forceinline__ void merge_wave()
     {
-#pragma unroll
-        for (int s = 32; s >= 1; s >>= 1) mx = fmaxf(mx, __shfl_xor(mx, s, 64));
+        mx = wave_fold(mx, [](float a, float b) { return fmaxf(a, b); });
         nan = __ballot(nan) != 0ull;
     }
     __device__ __forceinline__ float value() const { return nan ? u2f(kQNaN) : mx; }
@@ -688,9 +704,39 @@ __global__ __launch_bounds__(kThreads) void row_mean_kernel(const float* __restr
 }
 
 // ---------------------------------------------------------------- layer_norm forward (pam/pam_ops.py:350-378)
-template <int CH, class M, class L>
-__device__ __forceinline__ void layer_norm_row(float (&v)[CH], const float* __restrict__ weight, const float* __restrict__ bias,
-                                               L& lay, long n, float count, float eps, M& m)
+// The weight and bias elements of a lane are the same for every row it works on.  KEEP: they are read once and stay in
+// registers (rows of few values per lane, where a read per row and element -- each waited for where it is used, in the
+// middle of the row's chain -- was most of a row's time); else they are read per row, from cache.
+template <int CH, bool KEEP>
+struct RowParams {
+    const float* __restrict__ weight; const float* __restrict__ bias;
+    float w[KEEP ? CH : 1], b[KEEP ? CH : 1];
+    template <class L>
+    __device__ __forceinline__ void fetch(const L& lay, long n)
+    {
+        if constexpr (KEEP) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const long i = lay.index(c);
+                w[c] = (weight && i < n) ? weight[i] : 1.0f;
+                b[c] = (bias && i < n) ? bias[i] : 0.0f;
+            }
+        }
+    }
+    __device__ __forceinline__ float weight_at(int c, long i, bool inside) const
+    {
+        if constexpr (KEEP) return w[c]; else return inside ? weight[i] : 1.0f;
+    }
+    __device__ __forceinline__ float bias_at(int c, long i, bool inside) const
+    {
+        if constexpr (KEEP) return b[c]; else return inside ? bias[i] : 0.0f;
+    }
+};
+constexpr int kKeepForward = 16;       // values per lane up to which the forward kernels keep them (the gradient kernels have
+                                       // no registers to spare: with them kept, rows of 197 values ran 40 % slower)
+
+template <int CH, class M, class L, class P>
+__device__ __forceinline__ void layer_norm_row(float (&v)[CH], const P& par, L& lay, long n, float count, float eps, M& m)
 {
     // in place: inputs, then centred values, then results (one array of registers per row)
     float p = 0.0f;
@@ -710,8 +756,8 @@ __device__ __forceinline__ void layer_norm_row(float (&v)[CH], const float* __re
     for (int c = 0; c < CH; ++c) {
         const long i = lay.index(c); const bool inside = i < n;
         float r = m.div_by_positive(v[c], denom);                        // the centred value was recorded by square()
-        if (weight) r = m.mul_seen(r, inside ? weight[i] : 1.0f);
-        if (bias) r = r + (inside ? bias[i] : 0.0f);
+        if (par.weight) r = m.mul_seen(r, par.weight_at(c, i, inside));
+        if (par.bias) r = r + par.bias_at(c, i, inside);
         v[c] = r;
     }
 }
@@ -727,6 +773,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     float ahead[CH > 0 ? CH : 1];
     constexpr bool kAhead = false;                         // measured slower with it
     PAM_WAVE_FIRST_ROW(kAhead, ahead, x, 0.0f);
+    RowParams<(CH > 0 ? CH : 1), (CH > 0 && CH <= kKeepForward)> par{weight, bias};
+    if constexpr (CH > 0) par.fetch(WaveRow{lane}, n);
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
         if constexpr (CH > 0) {
@@ -734,10 +782,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             PAM_WAVE_NEXT_ROW(kAhead, v, ahead, x, 0.0f);
             WaveRow lay{lane};
             Unchecked u{o, Span()};
-            layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, u);
+            layer_norm_row<CH>(v, par, lay, n, count, eps, u);
             if (!wave_valid(u)) {                              // the row is read again (from cache)
                 load_row<CH>(v, xr, n, lane, 0.0f);
-                Checked k{o}; layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, k);
+                Checked k{o}; layer_norm_row<CH>(v, par, lay, n, count, eps, k);
             }
             store_row<CH>(v, yr, n, lay);
         } else {
@@ -985,9 +1033,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 
 // One row of the layer_norm gradient.  cen: x on entry, overwritten; g: dy on entry (1.0 past the
 // end), dx on exit; terms: the per-element terms of the weight gradient (if weight).
-template <int CH, class G, class L>
+template <int CH, class G, class L, class P>
 __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)[CH], float (&terms)[CH],
-                                                    const float* __restrict__ weight, L& lay, long n, float count, float eps, G& m)
+                                                    const P& par, L& lay, long n, float count, float eps, G& m)
 {
     float p = 0.0f;
 #pragma unroll
@@ -1008,8 +1056,8 @@ __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const long i = lay.index(c); const bool inside = i < n;
-        if (weight) {
-            const float xn = m.div(cen[c], denom), wi = inside ? weight[i] : 1.0f;
+        if (par.weight) {
+            const float xn = m.div(cen[c], denom), wi = par.weight_at(c, i, inside);
             terms[c] = m.mul_db(xn, wi, g[c]);
             g[c] = m.mul_da(xn, wi, g[c]);
         }
@@ -1130,6 +1178,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(((CH) 
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
     const float count = (float)n;
+    RowParams<CH, false> par{weight, nullptr};
     for (long r = wave; r < rows; r += nwaves) {
         float cen[CH], g[CH], terms[CH];
         bool done = false;
@@ -1138,14 +1187,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(((CH) 
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
             typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
-            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, u);
+            layer_norm_grad_row<CH>(cen, g, terms, par, lay, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
         if (!done) {                                    // the row is read again (from cache) rather than kept in registers
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
             GradChecked k{o, ap};
-            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, k);
+            layer_norm_grad_row<CH>(cen, g, terms, par, lay, n, count, eps, k);
         }
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
@@ -1283,16 +1332,18 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_fwd_b
     PAM_BLOCK_ROW_SETUP;
     const float count = (float)n;
     float ahead[CH];
-    constexpr bool kAhead = false;                         // measured slower with it
+    constexpr bool kAhead = CH < 16;                       // (rows of 10000 values: 91 -> 83 us for 4096 of them)
     PAM_BLOCK_FIRST_ROW(kAhead, ahead, x, 0.0f);
+    RowParams<CH, (CH <= kKeepForward)> par{weight, bias};
+    par.fetch(lay, n);
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float v[CH];
         PAM_BLOCK_NEXT_ROW(kAhead, v, ahead, x, 0.0f);
         Unchecked u{o, Span()};
-        layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, u);
+        layer_norm_row<CH>(v, par, lay, n, count, eps, u);
         if (!lay.all(u.valid())) {                             // the row is read again (from cache)
             load_row<CH>(v, x + r * n, n, lay, 0.0f);
-            Checked k{o}; layer_norm_row<CH>(v, weight, bias, lay, n, count, eps, k);
+            Checked k{o}; layer_norm_row<CH>(v, par, lay, n, count, eps, k);
         }
         store_row<CH>(v, y + r * n, n, lay);
     }
@@ -1330,6 +1381,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_bwd_b
 {
     PAM_BLOCK_ROW_SETUP;
     const float count = (float)n;
+    RowParams<CH, false> par{weight, nullptr};
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float cen[CH], g[CH], terms[CH];
         bool done = false;
@@ -1337,14 +1389,14 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_bwd_b
             load_row<CH>(cen, x + r * n, n, lay, 0.0f);
             load_row<CH>(g, gy + r * n, n, lay, 1.0f);
             typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
-            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, u);
+            layer_norm_grad_row<CH>(cen, g, terms, par, lay, n, count, eps, u);
             done = lay.all(u.valid());
         }
         if (!done) {                                    // the row is read again (from cache) rather than kept in registers
             load_row<CH>(cen, x + r * n, n, lay, 0.0f);
             load_row<CH>(g, gy + r * n, n, lay, 1.0f);
             GradChecked k{o, ap};
-            layer_norm_grad_row<CH>(cen, g, terms, weight, lay, n, count, eps, k);
+            layer_norm_grad_row<CH>(cen, g, terms, par, lay, n, count, eps, k);
         }
         store_row<CH>(g, dx + r * n, n, lay);
         if (weight && dw_terms) store_row<CH>(terms, dw_terms + r * n, n, lay);
