@@ -172,7 +172,14 @@ __device__ __forceinline__ float fold_shift(const float* __restrict__ partial, i
     __shared__ float fold_mx[WAVES];
     __shared__ int fold_nan[WAVES];
     MaxNan m;
-    for (int i = threadIdx.x; i < count; i += WAVES * 64) m.take(partial[i]);
+    // (all of a thread's loads in flight together: one after the other, each waited for, they were four cache
+    // latencies at the start of every work-group)
+    constexpr int kPer = (kMaxPartials + WAVES * 64 - 1) / (WAVES * 64);
+    float q[kPer];
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) { const int i = (int)threadIdx.x + u * WAVES * 64; q[u] = i < count ? partial[i] : u2f(0xff800000u); }
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) m.take(q[u]);
     m.merge_wave();
     if (threadIdx.x % 64 == 0) { fold_mx[threadIdx.x / 64] = m.mx; fold_nan[threadIdx.x / 64] = m.nan; }
     __syncthreads();
@@ -229,7 +236,13 @@ __device__ __forceinline__ float stream_sum(const float* __restrict__ p, long n,
         float a = p[i], b = p[i + 64], c = p[i + 128], d = p[i + 192];
         acc = acc + f(i, a); acc = acc + f(i + 64, b); acc = acc + f(i + 128, c); acc = acc + f(i + 192, d);
     }
-    for (; i < n; i += 64) acc = acc + f(i, p[i]);
+    // the ragged end: up to three more elements, their loads in flight together (one after the other, each waited
+    // for, they were most of the time of a row of 197 values)
+    const bool has_a = i < n, has_b = i + 64 < n, has_c = i + 128 < n;
+    const float a = has_a ? p[i] : 0.0f, b = has_b ? p[i + 64] : 0.0f, c = has_c ? p[i + 128] : 0.0f;
+    if (has_a) acc = acc + f(i, a);
+    if (has_b) acc = acc + f(i + 64, b);
+    if (has_c) acc = acc + f(i + 128, c);
     return acc;
 }
 
@@ -376,11 +389,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
-    const float shift = fold_shift<kWaves>(partial, partials);
-    if (wave == 0 && lane == 0) *shift_out = shift;
     float ahead[CH > 0 ? CH : 1];
     constexpr bool kAhead = CH >= 8;
-    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, kNegInf);                      // the fill has weight zero
+    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, kNegInf);                      // the fill has weight zero; in flight while the maxima are folded
+    const float shift = fold_shift<kWaves>(partial, partials);
+    if (wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; float* yr = y + r * n;
         float total;
@@ -653,11 +666,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 {
     const int lane = threadIdx.x % 64;
     const long wave = (long)blockIdx.x * kWaves + threadIdx.x / 64, nwaves = (long)gridDim.x * kWaves;
-    const float shift = fold_shift<kWaves>(partial, partials);
-    if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
     float ahead[CH > 0 ? CH : 1];
     constexpr bool kAhead = CH > 0;
-    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, 0.0f);
+    PAM_WAVE_FIRST_ROW(kAhead, ahead, x, 0.0f);                          // in flight while the maxima are folded
+    const float shift = fold_shift<kWaves>(partial, partials);
+    if (shift_out && wave == 0 && lane == 0) *shift_out = shift;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n;
         if constexpr (CH > 0) {
@@ -1238,11 +1251,11 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(C
                                                                          const float* __restrict__ partial, int partials)
 {
     PAM_BLOCK_ROW_SETUP;
-    const float shift = fold_shift<kBlockWaves>(partial, partials);
-    if (blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     float ahead[CH];
     constexpr bool kAhead = CH >= 16;
     PAM_BLOCK_FIRST_ROW(kAhead, ahead, x, kNegInf);
+    const float shift = fold_shift<kBlockWaves>(partial, partials);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float v[CH];
         PAM_BLOCK_NEXT_ROW(kAhead, v, ahead, x, kNegInf);
@@ -1290,11 +1303,11 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_block_
                                                                        Offset o, const float* __restrict__ partial, int partials)
 {
     PAM_BLOCK_ROW_SETUP;
-    const float shift = fold_shift<kBlockWaves>(partial, partials);
-    if (shift_out && blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     float ahead[CH];
     constexpr bool kAhead = CH < 16;                       // sixteen values per thread twice over would spill
     PAM_BLOCK_FIRST_ROW(kAhead, ahead, x, 0.0f);
+    const float shift = fold_shift<kBlockWaves>(partial, partials);
+    if (shift_out && blockIdx.x == 0 && threadIdx.x == 0) *shift_out = shift;
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float xv[CH];
         PAM_BLOCK_NEXT_ROW(kAhead, xv, ahead, x, 0.0f);
