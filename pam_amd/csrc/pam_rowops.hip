@@ -563,12 +563,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     const float shift = *shift_in;
     for (long r = wave; r < rows; r += nwaves) {
         const float* xr = x + r * n; const float* gr = dy + r * n; float* dr = dx + r * n;
-        const float total = row_sum[r];
-        const float inv = pad_div_off(1.0f, total, o.off, o.has);
         if constexpr (CH > 0) {
             float xv[CH], g[CH], out[CH];
             load_row<CH>(xv, xr, n, lane, kNegInf);
             load_row<CH>(g, gr, n, lane, 0.0f);
+            // (the row's total after the row's loads, and its reciprocal only where it is used: computed up here, it
+            // made every row wait for the total before its own loads were issued)
+            const float total = row_sum[r];
             bool done = false;
             WaveRow lay{lane};
             if (EXACT) {                                  // host: all exact, no offset
@@ -580,10 +581,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
                 done = wave_valid(u);
             }
-            if (!done) softmax_grad_row_checked<CH>(xv, g, out, total, inv, shift, lay, n, o, ap);
+            if (!done) softmax_grad_row_checked<CH>(xv, g, out, total, pad_div_off(1.0f, total, o.off, o.has), shift, lay, n, o, ap);
 #pragma unroll
             for (int c = 0; c < CH; ++c) { long i = lane + 64L * c; if (i < n) dr[i] = out[c]; }
         } else {
+            const float total = row_sum[r];
+            const float inv = pad_div_off(1.0f, total, o.off, o.has);
             bool done = false;
             if (EXACT) {                                  // the all-exact gradient as in softmax_grad_row_exact, in two sweeps
                 Unchecked m{o, Span()};
