@@ -271,26 +271,48 @@ struct Checked {
     __device__ __forceinline__ float div_by_positive(float a, float b) { return div(a, b); }
     __device__ __forceinline__ void record(float) {}
 };
-struct Unchecked {
+// OFFSETS: whether the chain carries the code for an offset.  Without it the chains are shorter; a call with an offset
+// then fails every row's check and its rows are redone with the checked functions (a test around the first attempt
+// instead cost the calls without an offset 5-15 % in the forward kernels).
+template <bool OFFSETS>
+struct UncheckedT {
     Offset o; Span sp;
-    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, o.has, sp); }
-    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, o.has, sp); }
-    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, o.has, sp); }
-    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, OFFSETS && o.has, sp); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, OFFSETS && o.has, sp); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, OFFSETS && o.has, sp); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, OFFSETS && o.has, sp); }
     __device__ __forceinline__ float log2_plain(float v) { return log2_entry_unchecked(v, 1.0f, false, sp); }
-    __device__ __forceinline__ float root(float v) { return pow_half_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float root(float v) { return pow_half_unchecked(v, o.off, OFFSETS && o.has, sp); }
     __device__ __forceinline__ float zero_over(float) { return 0.0f; }      // the divisor is a positive normal number when valid
-    __device__ __forceinline__ bool valid() const { return sp.normal(); }
+    __device__ __forceinline__ bool usable() const { return OFFSETS || !o.has; }         // (the same for every lane of a launch)
+    __device__ __forceinline__ bool valid() const { return usable() && sp.normal(); }
     // Cheaper forms (an offset takes the general ones).  mul_const: k is a positive normal constant; mul_seen and
     // div_by_positive: a was recorded earlier in the chain or is a result of exp2; div_by_positive: b is not negative
     // and was given to record().
-    __device__ __forceinline__ float mul_const(float a, float k) { return o.has ? mul(a, k) : pam_unchecked_const(a, k, sp); }
-    __device__ __forceinline__ float mul_seen(float a, float b) { return o.has ? mul(a, b) : pam_unchecked_seen(a, b, sp); }
-    __device__ __forceinline__ float square(float a) { return o.has ? mul(a, a) : pam_unchecked_square(a, sp); }
-    __device__ __forceinline__ float div_by_positive(float a, float b) { return o.has ? div(a, b) : pad_unchecked_by_positive(a, b, sp); }
+    __device__ __forceinline__ float mul_const(float a, float k) { return OFFSETS && o.has ? mul(a, k) : pam_unchecked_const(a, k, sp); }
+    __device__ __forceinline__ float mul_seen(float a, float b) { return OFFSETS && o.has ? mul(a, b) : pam_unchecked_seen(a, b, sp); }
+    __device__ __forceinline__ float square(float a) { return OFFSETS && o.has ? mul(a, a) : pam_unchecked_square(a, sp); }
+    __device__ __forceinline__ float div_by_positive(float a, float b) { return OFFSETS && o.has ? div(a, b) : pad_unchecked_by_positive(a, b, sp); }
     __device__ __forceinline__ void record(float v) { sp.see(f2u(v) & ~kSign); }
 };
-__device__ __forceinline__ bool wave_valid(const Unchecked& u) { return __ballot(!u.valid()) == 0ull; }
+template <bool OFFSETS>
+__device__ __forceinline__ bool wave_valid(const UncheckedT<OFFSETS>& u) { return __ballot(!u.valid()) == 0ull; }
+
+// Which kernel instances carry the offset's code in their unchecked first attempt: those where the shorter chains made
+// the compiler keep more in registers than the instance may have and spill (by measurement over every instance: the
+// others run 3-20 % faster without it).  BLOCK: a work-group per row.
+enum RowKernel { kSoftmaxFwd, kSoftmaxBwd, kSoftmaxBwdExact, kLogsumexpFwd, kLogsumexpBwd, kLayerNormFwd, kLayerNormBwd };
+template <RowKernel K, int CH, bool BLOCK>
+constexpr bool fast_path_offsets()
+{
+    if (K == kSoftmaxBwd || K == kSoftmaxBwdExact) return true;
+    if (K == kLayerNormBwd) return BLOCK ? CH >= 8 : CH == 12;
+    if (K == kLogsumexpBwd) return BLOCK ? CH >= 8 : (CH == 4 || CH == 12);
+    if (K == kLayerNormFwd) return !BLOCK && CH == 16;
+    if (K == kSoftmaxFwd) return BLOCK && (CH == 10 || CH == 12);
+    return false;                                                       // logsumexp forward
+}
+template <RowKernel K, int CH, bool BLOCK> using UncheckedFor = UncheckedT<fast_path_offsets<K, CH, BLOCK>()>;
 
 // ---------------------------------------------------------------- softmax forward (pam/pam_ops.py:305-328)
 __device__ __forceinline__ float softmax_weight(float x, float shift, Offset o)
@@ -401,7 +423,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             float v[CH];
             PAM_WAVE_NEXT_ROW(kAhead, v, ahead, x, kNegInf);
             WaveRow lay{lane};
-            Unchecked u{o, Span()};
+            UncheckedFor<kSoftmaxFwd, CH, false> u{o, Span()};
             total = softmax_row<CH>(v, shift, u, lay);
             if (!wave_valid(u)) {                              // the row is read again (from cache)
                 load_row<CH>(v, xr, n, lane, kNegInf);
@@ -409,7 +431,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             }
             store_row<CH>(v, yr, n, lay);
         } else {
-            Unchecked u{o, Span()};
+            UncheckedFor<kSoftmaxFwd, CH, false> u{o, Span()};
             total = softmax_stream(xr, yr, n, lane, shift, u);
             if (!wave_valid(u)) { Checked k{o}; total = softmax_stream(xr, yr, n, lane, shift, k); }
         }
@@ -449,9 +471,9 @@ __device__ __forceinline__ float softmax_dx(float xv, float e, float g, float in
 // The all-approximate gradient of one register-resident row with unchecked arithmetic.  Masked
 // (-inf) elements and the lanes past the end of the row are computed on a stand-in value and
 // replaced by the zeros the chain gives them.
-template <int CH, class L>
+template <int CH, class L, class U>
 __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
-                                                        float total, float shift, L& lay, long n, Unchecked& m)
+                                                        float total, float shift, L& lay, long n, U& m)
 {
     const float inv = m.div(1.0f, total);
     float e[CH];
@@ -486,9 +508,9 @@ __device__ __forceinline__ void softmax_grad_row_approx(const float (&xv)[CH], c
 // masked to sign and exponent; the quotient's gradient for its divisor is -(2^e(a (/) b) / 2^e(b)) g, a difference of
 // exponent fields; exp2's is 2^e(exp2 t) g.  The products with the upstream gradients are IEEE products in both
 // forms, so those gradients need no recording; everything else is recorded as in the approximate chain.
-template <int CH, class L>
+template <int CH, class L, class U>
 __device__ __forceinline__ void softmax_grad_row_exact(const float (&xv)[CH], const float (&g)[CH], float (&out)[CH],
-                                                       float total, float shift, L& lay, long n, Unchecked& m)
+                                                       float total, float shift, L& lay, long n, U& m)
 {
     const uint32_t tot = f2u(total);
     m.record(total);                                                       // a sum of weights: never negative
@@ -573,11 +595,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             bool done = false;
             WaveRow lay{lane};
             if (EXACT) {                                  // host: all exact, no offset
-                Unchecked u{o, Span()};
+                UncheckedFor<kSoftmaxBwdExact, CH, false> u{o, Span()};
                 softmax_grad_row_exact<CH>(xv, g, out, total, shift, lay, n, u);
                 done = wave_valid(u);
             } else if (ap.a && ap.b && ap.e) {            // the all-approximate gradient has an unchecked form
-                Unchecked u{o, Span()};
+                UncheckedFor<kSoftmaxBwd, CH, false> u{o, Span()};
                 softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
                 done = wave_valid(u);
             }
@@ -589,7 +611,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             const float inv = pad_div_off(1.0f, total, o.off, o.has);
             bool done = false;
             if (EXACT) {                                  // the all-exact gradient as in softmax_grad_row_exact, in two sweeps
-                Unchecked m{o, Span()};
+                UncheckedFor<kSoftmaxBwdExact, CH, false> m{o, Span()};
                 const uint32_t tot = f2u(total), inv_b = kBias - tot + kBias, slope_c = f2u(kLog2E);
                 m.record(total); m.sp.see(inv_b); m.sp.see(inv_b + 0x00800000u);
                 auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul_const(masked ? 1.0f : x, kLog2E) - shift); };
@@ -614,7 +636,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 });
                 done = wave_valid(m);
             } else if (ap.a && ap.b && ap.e) {            // the all-approximate gradient, branch-free forms first
-                Unchecked m{o, Span()};
+                UncheckedFor<kSoftmaxBwd, CH, false> m{o, Span()};
                 const float inv_u = m.div(1.0f, total);
                 auto weight = [&](float x, bool masked) { return m.exp2(masked ? 0.5f : m.mul(masked ? 1.0f : x, kLog2E) - shift); };
                 float p = 0.0f;
@@ -680,7 +702,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             float xv[CH];
             PAM_WAVE_NEXT_ROW(kAhead, xv, ahead, x, 0.0f);
             WaveRow lay{lane};
-            Unchecked u{o, Span()};
+            UncheckedFor<kLogsumexpFwd, CH, false> u{o, Span()};
             float out = logsumexp_row<CH>(xv, shift, lay, n, u);
             if (!wave_valid(u)) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lay, n, k); }
             if (lse && lane == 0) lse[r] = out;
@@ -697,7 +719,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                 });
                 return m.div(shift + m.log2_plain(wave_sum(p)), kLog2E);
             };
-            Unchecked u{o, Span()};
+            UncheckedFor<kLogsumexpFwd, CH, false> u{o, Span()};
             float out = sweep(u);
             if (!wave_valid(u)) { Checked k{o}; out = sweep(k); }
             if (lse && lane == 0) lse[r] = out;
@@ -797,7 +819,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
             float v[CH];
             PAM_WAVE_NEXT_ROW(kAhead, v, ahead, x, 0.0f);
             WaveRow lay{lane};
-            Unchecked u{o, Span()};
+            UncheckedFor<kLayerNormFwd, CH, false> u{o, Span()};
             layer_norm_row<CH>(v, par, lay, n, count, eps, u);
             if (!wave_valid(u)) {                              // the row is read again (from cache)
                 load_row<CH>(v, xr, n, lane, 0.0f);
@@ -823,7 +845,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
                     if (inside) yr[i] = r;
                 });
             };
-            Unchecked u{o, Span()};
+            UncheckedFor<kLayerNormFwd, CH, false> u{o, Span()};
             sweep(u);
             if (!wave_valid(u)) { Checked k{o}; sweep(k); }
         }
@@ -835,7 +857,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 // 262-276 for the formulas; pam/pam_ops.py:331-378 for the ops).  Rows of up to 1024 values stay in
 // registers; longer rows are swept several times (the later sweeps find the row in cache).
 // GradChecked serves every combination of exact and approximate gradients;
-// GradUnchecked is the all-approximate chain on the branch-free primitives, tried first and kept
+// GradUncheckedT is the all-approximate chain on the branch-free primitives, tried first and kept
 // when every value it touched was a normal number.
 struct GradChecked {
     Offset o; Approx ap;
@@ -868,12 +890,13 @@ __device__ __forceinline__ float log2_exact_dx_unchecked(float x, float g, Span&
     sp.see(xi); sp.see(xi + 0x00800000u);
     return u2f((254u << 23) - (xi & kExpo)) * g;
 }
-struct GradUnchecked {
+template <bool OFFSETS>
+struct GradUncheckedT {
     Offset o; Span sp;
-    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, o.has, sp); }
-    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, o.has, sp); }
-    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, o.has, sp); }
-    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, o.has, sp); }
+    __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, OFFSETS && o.has, sp); }
+    __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, OFFSETS && o.has, sp); }
+    __device__ __forceinline__ float exp2(float t) { return exp2_entry_unchecked(t, o.off, OFFSETS && o.has, sp); }
+    __device__ __forceinline__ float log2(float v) { return log2_entry_unchecked(v, o.off, OFFSETS && o.has, sp); }
     __device__ __forceinline__ float mul_da(float, float b, float g) { return mul(g, b); }
     __device__ __forceinline__ float mul_db(float a, float, float g) { return mul(g, a); }
     __device__ __forceinline__ float div_da(float, float b, float g) { return mul(div(1.0f, b), g); }
@@ -882,8 +905,10 @@ struct GradUnchecked {
     __device__ __forceinline__ float log2_dx(float x, float g) { return div(div(g, x), kLn2); }
     __device__ __forceinline__ float log2_plain(float v) { return log2_entry_unchecked(v, 1.0f, false, sp); }
     __device__ __forceinline__ float log2_plain_dx(float x, float g) { return log2_exact_dx_unchecked(x, g, sp); }
-    __device__ __forceinline__ bool valid() const { return sp.normal(); }
+    __device__ __forceinline__ bool usable() const { return OFFSETS || !o.has; }         // (the same for every lane of a launch)
+    __device__ __forceinline__ bool valid() const { return usable() && sp.normal(); }
 };
+template <RowKernel K, int CH, bool BLOCK> using GradUncheckedFor = GradUncheckedT<fast_path_offsets<K, CH, BLOCK>()>;
 
 // The all-exact gradients (the reference's default) without an offset, on unchecked arithmetic.  In the normal range
 // the exact backward formulas are short (pam/cuda_kernels.cu:40-58, 85-97, 115-123, 132-136): the gradient of a (*) b
@@ -916,6 +941,7 @@ struct GradUncheckedExact {
     __device__ __forceinline__ float log2_dx(float x, float g) { return log2_exact_dx_unchecked(x, g, sp); }
     __device__ __forceinline__ float log2_plain(float v) { return log2(v); }
     __device__ __forceinline__ float log2_plain_dx(float x, float g) { return log2_dx(x, g); }
+    __device__ __forceinline__ bool usable() const { return true; }
     __device__ __forceinline__ bool valid() const { return sp.normal(); }
 };
 
@@ -967,7 +993,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         bool done = false;
         WaveRow lay{lane};
         if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
-            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUncheckedFor<kLogsumexpBwd, CH, false>>::type u{o, Span()};
             logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1039,7 +1065,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
         if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
-            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUncheckedFor<kLogsumexpBwd, 0, false>>::type u{o, Span()};
             logsumexp_grad_stream(x + r * n, gr, dx + r * n, g_row, log_softmax != 0, shift, lane, n, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1175,7 +1201,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
         float* tr = (weight && dw_terms) ? dw_terms + r * n : nullptr;
         bool done = false;
         if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
-            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUncheckedFor<kLayerNormBwd, 0, false>>::type u{o, Span()};
             layer_norm_grad_stream(x + r * n, gy + r * n, weight, dx + r * n, tr, lane, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1202,7 +1228,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(((CH) 
         if (EXACT || (ap.a && ap.b && ap.e)) {
             load_row<CH>(cen, x + r * n, n, lane, 0.0f);
             load_row<CH>(g, gy + r * n, n, lane, 1.0f);
-            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUncheckedFor<kLayerNormBwd, CH, false>>::type u{o, Span()};
             layer_norm_grad_row<CH>(cen, g, terms, par, lay, n, count, eps, u);
             done = __ballot(!u.valid()) == 0ull;
         }
@@ -1262,7 +1288,7 @@ __global__ __launch_bounds__(kBlockThreads) __attribute__((amdgpu_waves_per_eu(C
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float v[CH];
         PAM_BLOCK_NEXT_ROW(kAhead, v, ahead, x, kNegInf);
-        Unchecked u{o, Span()};
+        UncheckedFor<kSoftmaxFwd, CH, true> u{o, Span()};
         float total = softmax_row<CH>(v, shift, u, lay);
         if (!lay.all(u.valid())) {                             // the row is read again (from cache)
             load_row<CH>(v, x + r * n, n, lay, kNegInf);
@@ -1287,11 +1313,11 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void softmax_bwd_bloc
         load_row<CH>(g, dy + r * n, n, lay, 0.0f);
         bool done = false;
         if (EXACT) {
-            Unchecked u{o, Span()};
+            UncheckedFor<kSoftmaxBwdExact, CH, true> u{o, Span()};
             softmax_grad_row_exact<CH>(xv, g, out, total, shift, lay, n, u);
             done = lay.all(u.valid());
         } else if (ap.a && ap.b && ap.e) {
-            Unchecked u{o, Span()};
+            UncheckedFor<kSoftmaxBwd, CH, true> u{o, Span()};
             softmax_grad_row_approx<CH>(xv, g, out, total, shift, lay, n, u);
             done = lay.all(u.valid());
         }
@@ -1314,7 +1340,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_block_
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float xv[CH];
         PAM_BLOCK_NEXT_ROW(kAhead, xv, ahead, x, 0.0f);
-        Unchecked u{o, Span()};
+        UncheckedFor<kLogsumexpFwd, CH, true> u{o, Span()};
         float out = logsumexp_row<CH>(xv, shift, lay, n, u);
         if (!lay.all(u.valid())) { Checked k{o}; out = logsumexp_row<CH>(xv, shift, lay, n, k); }
         if (lse && threadIdx.x == 0) lse[r] = out;
@@ -1355,7 +1381,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_fwd_b
     for (long r = blockIdx.x; r < rows; r += gridDim.x) {
         float v[CH];
         PAM_BLOCK_NEXT_ROW(kAhead, v, ahead, x, 0.0f);
-        Unchecked u{o, Span()};
+        UncheckedFor<kLayerNormFwd, CH, true> u{o, Span()};
         layer_norm_row<CH>(v, par, lay, n, count, eps, u);
         if (!lay.all(u.valid())) {                             // the row is read again (from cache)
             load_row<CH>(v, x + r * n, n, lay, 0.0f);
@@ -1381,7 +1407,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void logsumexp_bwd_bl
         const float g_row = log_softmax ? 0.0f : grad[r];
         bool done = false;
         if (EXACT || (ap.a && ap.b && ap.e)) {         // EXACT: the host chose this instance for all-exact gradients without an offset
-            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUncheckedFor<kLogsumexpBwd, CH, true>>::type u{o, Span()};
             logsumexp_grad_row<CH>(xv, gy, out, g_row, log_softmax != 0, shift, lay, n, u);
             done = lay.all(u.valid());
         }
@@ -1404,7 +1430,7 @@ __global__ __launch_bounds__(kBlockThreads) PAM_BLOCK_ATTR void layer_norm_bwd_b
         if (EXACT || (ap.a && ap.b && ap.e)) {
             load_row<CH>(cen, x + r * n, n, lay, 0.0f);
             load_row<CH>(g, gy + r * n, n, lay, 1.0f);
-            typename std::conditional<EXACT, GradUncheckedExact, GradUnchecked>::type u{o, Span()};
+            typename std::conditional<EXACT, GradUncheckedExact, GradUncheckedFor<kLayerNormBwd, CH, true>>::type u{o, Span()};
             layer_norm_grad_row<CH>(cen, g, terms, par, lay, n, count, eps, u);
             done = lay.all(u.valid());
         }
