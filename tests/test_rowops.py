@@ -337,8 +337,9 @@ def _dev(a):
 @pytest.mark.parametrize("off", [None, OFF])
 def test_gpu_softmax_forward_backward(oracle, off):
     # 4097 ... 16384 values: a work-group per row
-    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (64, 197), (7, 300), (7, 384), (2, 1000), (300, 32), (3, 4096), (5, 4097), (3, 6145), (2, 10000),
-                    (2, 16384), (2, 16385)]:
+    # (every values-per-lane instance of the register-resident kernels: 64, 65, 192, 197, 300, 512, 768, 1000)
+    for rows, n in [(1, 1), (3, 5), (4, 63), (4, 64), (5, 65), (5, 192), (64, 197), (7, 300), (7, 384), (3, 512), (3, 768), (2, 1000), (300, 32), (3, 4096), (5, 4097),
+                    (3, 6145), (2, 10000), (2, 12288), (2, 16384), (2, 16385)]:
         x = rows_case(rows * 1000 + n, rows, n)
         g = np.random.RandomState(n).standard_normal(x.shape).astype(np.float32)
         want, row_sum, shift = oracle.softmax_fwd(x, off)
