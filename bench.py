@@ -390,6 +390,23 @@ def main():
             "sample": f"fwd + dX + dW of the 192->768 layer (5.58 G PAM-MAC), {reps} times in about 10 s, this repository's C "
                       "restatement (integer add + fp32 accumulate, OpenMP over rows), contiguous operands",
         }
+        # A second figure beside it: the reference's class of CPU algorithm (float log2 / add / exp2 on tensors, every
+        # product of the matrix product materialised and then summed) on its own CPU-runnable case, 256 x 512 x 256
+        # (benchmark configuration 0): forward and the two products of the approximate backward, median of 5.
+        from oracle import float_chain
+        gc = torch.Generator(device="cpu").manual_seed(0)
+        A0, B0, dY0 = torch.randn(256, 512, generator=gc), torch.randn(512, 256, generator=gc), torch.randn(256, 256, generator=gc)
+        float_chain.pam_matmul(A0, B0)
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            float_chain.pam_matmul(A0, B0); float_chain.pam_matmul(dY0, B0.T); float_chain.pam_matmul(A0.T, dY0)
+            times.append(time.perf_counter() - t0)
+        out["cpu_baseline"]["float_chain"] = {
+            "value": round(3 * 256 * 512 * 256 / sorted(times)[2] / 1e9, 3), "unit": "GMAC/s", "cores": torch.get_num_threads(),
+            "sample": "fwd + dX + dW at 256 x 512 x 256 (0.1 G PAM-MAC), median of 5, torch CPU float chain with the n x k x m "
+                      "products materialised (oracle/float_chain.py)",
+        }
     print(json.dumps(out))
 
 

@@ -247,3 +247,23 @@ def test_gemm_bruteforce_and_orders(oracle):
                 acc = np.float32(acc + oracle.pam_bwd(D[i, j:j + 1], A[i, k:k + 1], B[k:k + 1, j])[0])
             want[i, j] = acc
     assert_same_bits(got, want, "exact bwd delta_R")
+
+
+def test_float_chain_baseline_agrees_with_the_integer_definition(oracle):
+    """The torch float-chain restatement that bench.py times as its second CPU baseline (the reference's class of CPU
+    algorithm: float log2 / add / exp2, all products materialised) against the exact oracle: powers of two exactly,
+    full mantissas to the rounding of the fp32 log2 sum (a few 1e-7 of the largest sum)."""
+    import torch
+    from oracle import float_chain
+    rng = np.random.RandomState(5)
+    a = rng.standard_normal((24, 40)).astype(np.float32); b = rng.standard_normal((40, 28)).astype(np.float32)
+    a[3, 5] = 0.0; b[7, 2] = -0.0
+    got = float_chain.pam_matmul(torch.from_numpy(a), torch.from_numpy(b)).numpy()
+    want = oracle.gemm(a, b)
+    assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max()
+    p2a = np.ldexp(1.0, rng.randint(-8, 8, (6, 9))).astype(np.float32) * rng.choice([-1.0, 1.0], (6, 9)).astype(np.float32)
+    p2b = np.ldexp(1.0, rng.randint(-8, 8, (9, 5))).astype(np.float32)
+    assert_same_bits(float_chain.pam_matmul(torch.from_numpy(p2a), torch.from_numpy(p2b)).numpy(), p2a @ p2b, "powers of two")
+    x = rng.standard_normal(4096).astype(np.float32); y = rng.standard_normal(4096).astype(np.float32)
+    e = float_chain.pam(torch.from_numpy(x), torch.from_numpy(y)).numpy()
+    assert np.abs(e - oracle.pam(x, y)).max() <= 2e-6 * np.abs(e).max()
