@@ -105,6 +105,10 @@ def test_conv2d_composition(on_cpu):
     assert conv(Xg).shape == (2, 16, 7, 6)
     with pytest.raises(ValueError):
         pam_amd.conv2d(X, W, padding="circular")
+    # a dilation other than 1: the reference sizes its output without it (pam/pam_ops.py:137-138) and its final view
+    # of the unfolded product raises; the same here
+    with pytest.raises(RuntimeError):
+        pam_amd.conv2d(X, W, None, dilation=2)
 
 
 def _close(a, b):
