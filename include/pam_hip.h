@@ -197,9 +197,11 @@ int pam_hip_layer_norm_bwd(const float *x, const float *weight, const float *dy,
  * image patches read in place: x[batch][c][h][w] and w[co][c][kh][kw] contiguous, dilation 1,
  * output size (in + 2 pad - k) / stride + 1.  groups > 1 is the grouped convolution of
  * pam.conv2d_group (:163-198): w[co][c / groups][kh][kw], channels and filters fall into groups that
- * do not mix, one product per group on the same kernel (groups = 1 otherwise).  Sums run over
- * k = (c, i, j) of the group in ascending order in the chunks
- * pam_hip_gemm_plan(batch, co / groups, ho*wo, (c / groups)*kh*kw) reports. */
+ * do not mix (groups = 1 otherwise); one launch covers all (image, group) pairs, with one copy of the
+ * weights per image in the workspace where a product reads them -- unless those copies would exceed
+ * 32 MiB, then one launch per group.  Sums run over k = (c, i, j) of the group in ascending order in
+ * the chunks pam_hip_gemm_plan(batch * groups, co / groups, ho*wo, (c / groups)*kh*kw) reports
+ * (batch in place of batch * groups for a product that is launched per group). */
 size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,
                                       long stride_h, long stride_w, long pad_h, long pad_w, long groups, int which, float offset);
 /* which: 0 forward, 1 weight gradient, 2 input gradient */

@@ -1,5 +1,6 @@
 // PAM matrix products for gfx950, host side: the plan of a launch, the entry points of the C ABI for products and
 // convolutions, and the scratch the library owns.  The kernel is in pam_gemm_kernel.h.
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstring>
@@ -289,23 +290,36 @@ __global__ __launch_bounds__(256) void conv_tables_kernel(int2* __restrict__ kta
     }
 }
 
-__global__ __launch_bounds__(256) void scale_kernel(const float* __restrict__ in, float* __restrict__ out, size_t n, float off)
+// out = `copies` copies of in[0 .. n), each value (*) off if has_off
+__global__ __launch_bounds__(256) void scale_kernel(const float* __restrict__ in, float* __restrict__ out, size_t n, size_t copies, float off,
+                                                    int has_off)
 {
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) out[i] = pam_mul(in[i], off);
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n * copies; i += (size_t)gridDim.x * 256) {
+        const float v = in[i % n];
+        out[i] = has_off ? pam_mul(v, off) : v;
+    }
+}
+void launch_scale(const float* in, float* out, size_t n, size_t copies, float off, bool has_off, hipStream_t st)
+{
+    size_t blocks = (n * copies + 1023) / 1024;
+    if (blocks > (1u << 20)) blocks = 1u << 20;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, in, out, n, copies, off, has_off ? 1 : 0);
 }
 
 // wf[c][co][i][j] = w[co][c][kh-1-i][kw-1-j] (*) off: the weights of the convolution over the
 // upstream gradient that yields the gradient of the input (stride 1)
 // (with groups: c runs over all channels, co over the filters of c's group, and w is [filters][c per group][kh][kw])
+// (`copies` of them one after the other: see kReplicateBytes)
 __global__ __launch_bounds__(256) void flip_weights_kernel(const float* __restrict__ w, float* __restrict__ wf, int c, int cog, int cg, int kh, int kw,
-                                                          float off, int has_off)
+                                                          float off, int has_off, int copies)
 {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    if (idx >= c * cog * kh * kw) return;
+    const long at = (long)blockIdx.x * 256 + threadIdx.x, n = (long)c * cog * kh * kw;
+    if (at >= n * copies) return;
+    const int idx = (int)(at % n);
     const int j = idx % kw, i = (idx / kw) % kh, o = (idx / (kw * kh)) % cog, ci = idx / (kw * kh * cog);
     const int filter = (ci / cg) * cog + o;
     const float v = w[(((long)filter * cg + ci % cg) * kh + (kh - 1 - i)) * kw + (kw - 1 - j)];
-    wf[idx] = has_off ? pam_mul(v, off) : v;
+    wf[at] = has_off ? pam_mul(v, off) : v;
 }
 
 size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
@@ -324,16 +338,29 @@ int conv_shape(const char* what, ConvShape& s)
     return PAM_HIP_OK;
 }
 
-// workspace: [k table][l table][operand scaled by the offset, if any][split-k partial tiles]
+// A grouped convolution is one launch over (image, group) pairs: unit z = image * groups + group finds its rows of the
+// image, of the upstream gradient and of the output at z times one group's size, since an image's groups lie one after
+// the other.  Only the weights do not follow that pattern (every image uses all of them), so where a product reads them
+// it gets one copy per image -- up to this many bytes of copies; beyond, the groups are launched one by one.
+constexpr size_t kReplicateBytes = 32u << 20;
+bool replicated(const ConvShape& s) { return s.g > 1 && (size_t)s.batch * s.co * s.K() * sizeof(float) <= kReplicateBytes; }
+
+// workspace: [k table][l table][operand scaled by the offset, or the weights' copies, if any][split-k partial tiles]
+// which: 0 forward, 1 weight gradient approximate, 2 weight gradient exact
 struct ConvSpace { size_t tables, scaled, total; };
-ConvSpace conv_space(const ConvShape& s, bool weight_gradient, bool has_off)
+ConvSpace conv_space(const ConvShape& s, int which, bool has_off)
 {
     ConvSpace w;
     w.tables = align256((size_t)(s.K() + s.L()) * sizeof(int2));
-    size_t scaled_elems = !has_off ? 0 : weight_gradient ? (size_t)s.batch * s.co * s.L() : (size_t)s.co * s.K();
+    const size_t copies = replicated(s) ? (size_t)s.batch : 1;
+    size_t scaled_elems = 0;
+    if (which == 0) scaled_elems = (has_off || copies > 1) ? copies * s.co * s.K() : 0;
+    else if (which == 1) scaled_elems = has_off ? (size_t)s.batch * s.co * s.L() : 0;
+    else scaled_elems = copies > 1 ? copies * s.co * s.K() : 0;
     w.scaled = align256(scaled_elems * sizeof(float));
-    size_t split = weight_gradient ? pam_hip_gemm_workspace_bytes(s.batch, s.cog(), s.K(), s.L())
-                                   : pam_hip_gemm_workspace_bytes(s.batch, s.cog(), s.L(), s.K());
+    const long launches = s.g > 1 && (which == 1 || replicated(s)) ? s.batch * s.g : s.batch;
+    size_t split = which != 0 ? pam_hip_gemm_workspace_bytes(launches, s.cog(), s.K(), s.L())
+                              : pam_hip_gemm_workspace_bytes(launches, s.cog(), s.L(), s.K());
     w.total = w.tables + w.scaled + split;
     return w;
 }
@@ -372,8 +399,9 @@ ConvSpace input_gradient_space(const ConvShape& t)
 {
     ConvSpace w;
     w.tables = align256((size_t)(t.K() + t.L()) * sizeof(int2));
-    w.scaled = align256((size_t)t.co * t.K() * sizeof(float));
-    w.total = w.tables + w.scaled + pam_hip_gemm_workspace_bytes(t.batch, t.cog(), t.L(), t.K());
+    const bool copies = replicated(t);
+    w.scaled = align256((copies ? (size_t)t.batch : 1) * t.co * t.K() * sizeof(float));
+    w.total = w.tables + w.scaled + pam_hip_gemm_workspace_bytes(copies ? t.batch * t.g : t.batch, t.cog(), t.L(), t.K());
     return w;
 }
 
@@ -510,7 +538,9 @@ size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long c
         if (input_gradient_shape("conv2d_workspace_bytes", s, t) != PAM_HIP_OK) return 0;
         return input_gradient_space(t).total;
     }
-    return conv_space(s, which != 0, offset != 1.0f).total;
+    // (1: the larger of the two weight gradients' needs, whichever the caller then asks for)
+    if (which == 1) return std::max(conv_space(s, 1, offset != 1.0f).total, conv_space(s, 2, false).total);
+    return conv_space(s, 0, offset != 1.0f).total;
 }
 
 int pam_hip_conv2d_bwd_input(const float* dy, const float* w, const float* x, float* dx, long batch, long c, long h, long wd,
@@ -531,13 +561,22 @@ int pam_hip_conv2d_bwd_input(const float* dy, const float* w, const float* x, fl
     rc = conv_prepare("conv2d_bwd_input", t, sp, workspace, workspace_bytes, st, cv, false);
     if (rc != PAM_HIP_OK) return rc;
     float* wf = (float*)((char*)workspace + sp.tables);
-    const long n = c * s.cog() * kh * kw;
+    const bool one_launch = replicated(t);
+    const long copies = one_launch ? batch : 1;
+    const long n = c * s.cog() * kh * kw * copies;
     // approximate: the offset goes into the flipped weights; exact: the product kernel applies it to its slope operand
     hipLaunchKernelGGL(flip_weights_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w, wf, (int)c, (int)s.cog(), (int)s.cg(),
-                       (int)kh, (int)kw, offset, (!exact && offset != 1.0f) ? 1 : 0);
+                       (int)kh, (int)kw, offset, (!exact && offset != 1.0f) ? 1 : 0, (int)copies);
     const long K = t.K(), L = t.L();                  // K = (co / groups) kh kw, L = h w
     void* rest = (char*)workspace + sp.tables + sp.scaled; size_t rest_bytes = workspace_bytes - sp.tables - sp.scaled;
     const long hw_out = s.ho * s.wo;
+    if (one_launch) {                                 // unit z = image * groups + group (see kReplicateBytes)
+        if (exact)
+            return gemm("conv2d_bwd_input", MODE_BWD_DR, batch * groups, s.cg(), L, K, wf, s.cg() * K, K, 1, dy, s.cog() * hw_out, 0, 0,
+                        x, s.cg() * L, L, 1, dx, s.cg() * L, L, 1, offset, rest, rest_bytes, stream, &cv);
+        return gemm("conv2d_bwd_input", MODE_PAM, batch * groups, s.cg(), L, K, wf, s.cg() * K, K, 1, dy, s.cog() * hw_out, 0, 0,
+                    nullptr, 0, 0, 0, dx, s.cg() * L, L, 1, 1.0f, rest, rest_bytes, stream, &cv);
+    }
     for (long gi = 0; gi < groups; ++gi) {            // one product per group: its filters' gradient slices in, its channels out
         const float* wg = wf + gi * s.cg() * K;
         const float* dyg = dy + gi * s.cog() * hw_out;
@@ -564,20 +603,24 @@ int pam_hip_conv2d_fwd(const float* x, const float* w, float* y, long batch, lon
     if (!x || !w || !y) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_fwd: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const bool has_off = offset != 1.0f;
-    ConvSpace sp = conv_space(s, false, has_off);
+    ConvSpace sp = conv_space(s, 0, has_off);
     ConvGeom cv;
     rc = conv_prepare("conv2d_fwd", s, sp, workspace, workspace_bytes, st, cv, false);
     if (rc != PAM_HIP_OK) return rc;
     // the reference folds the offset into the weights (the right operand of its product); here the
     // weights are the left operand, so they are scaled once up front
     const float* wl = w;
-    if (has_off) {
+    const bool one_launch = replicated(s);
+    if (has_off || one_launch) {
         float* scaled = (float*)((char*)workspace + sp.tables);
-        size_t n = (size_t)co * s.K();
-        hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, st, w, scaled, n, offset);
+        launch_scale(w, scaled, (size_t)co * s.K(), one_launch ? (size_t)batch : 1, offset, has_off, st);
         wl = scaled;
     }
     const long K = s.K(), L = s.L();
+    if (one_launch)                                   // unit z = image * groups + group (see kReplicateBytes)
+        return gemm("conv2d_fwd", MODE_PAM, batch * groups, s.cog(), L, K, wl, s.cog() * K, K, 1, x, s.cg() * h * wd, 0, 0,
+                    nullptr, 0, 0, 0, y, s.cog() * L, L, 1, 1.0f,
+                    (char*)workspace + sp.tables + sp.scaled, workspace_bytes - sp.tables - sp.scaled, stream, &cv);
     // per image and group: Y[co, l] = sum_k W[co, k] (*) patches[k, l] over the group's channels
     for (long gi = 0; gi < groups; ++gi) {
         rc = gemm("conv2d_fwd", MODE_PAM, batch, s.cog(), L, K, wl + gi * s.cog() * K, 0, K, 1, x + gi * s.cg() * h * wd, c * h * wd, 0, 0,
@@ -599,7 +642,7 @@ int pam_hip_conv2d_bwd_weight(const float* x, const float* dy, const float* w, f
     if (!x || !dy || !dw || (exact && !w)) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_bwd_weight: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const bool scale = offset != 1.0f && !exact;
-    ConvSpace sp = conv_space(s, true, scale);
+    ConvSpace sp = conv_space(s, exact ? 2 : 1, scale);
     ConvGeom cv;
     rc = conv_prepare("conv2d_bwd_weight", s, sp, workspace, workspace_bytes, st, cv, true);
     if (rc != PAM_HIP_OK) return rc;
@@ -609,10 +652,18 @@ int pam_hip_conv2d_bwd_weight(const float* x, const float* dy, const float* w, f
     const float* dl = dy;
     if (scale) {
         float* scaled = (float*)((char*)workspace + sp.tables);
-        size_t n = (size_t)batch * co * L;
-        size_t blocks = (n + 1023) / 1024; if (blocks > (1u << 20)) blocks = 1u << 20;
-        hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, st, dy, scaled, n, offset);
+        launch_scale(dy, scaled, (size_t)batch * co * L, 1, offset, true, st);
         dl = scaled;
+    }
+    // grouped: unit z = image * groups + group (see kReplicateBytes); only the exact gradient reads the weights
+    if (groups > 1 && !exact)
+        return gemm("conv2d_bwd_weight", MODE_PAM, batch * groups, s.cog(), K, L, dl, s.cog() * L, L, 1, x, s.cg() * h * wd, 0, 0,
+                    nullptr, 0, 0, 0, dw, s.cog() * K, K, 1, 1.0f, rest, rest_bytes, stream, &cv);
+    if (groups > 1 && replicated(s)) {
+        float* copies = (float*)((char*)workspace + sp.tables);
+        launch_scale(w, copies, (size_t)co * K, (size_t)batch, 1.0f, false, st);
+        return gemm("conv2d_bwd_weight", MODE_BWD_DL, batch * groups, s.cog(), K, L, dy, s.cog() * L, L, 1, x, s.cg() * h * wd, 0, 0,
+                    copies, s.cog() * K, K, 1, dw, s.cog() * K, K, 1, offset, rest, rest_bytes, stream, &cv);
     }
     for (long gi = 0; gi < groups; ++gi) {
         const float* xg = x + gi * s.cg() * h * wd;

@@ -225,9 +225,9 @@ def test_grouped_convolution_against_oracle(oracle, case, off):
         K = P.shape[1]
         W2 = Wg.reshape(cog, K)
         Wl = W2 if off is None else oracle.pam(W2, np.float32(off))
-        want = oracle.gemm(np.broadcast_to(Wl, (batch, cog, K)), P, kchunk=_plan(batch, cog, L, K))
+        want = oracle.gemm(np.broadcast_to(Wl, (batch, cog, K)), P, kchunk=_plan(batch * G, cog, L, K))          # one launch over (image, group) pairs
         assert_same_bits(Y[:, g * cog:(g + 1) * cog].cpu().numpy().reshape(batch, cog, L), want, f"grouped forward, group {g}")
-        Pt = np.ascontiguousarray(P.transpose(0, 2, 1)); d2 = dYg.reshape(batch, cog, L); plan = _plan(batch, cog, K, L)
+        Pt = np.ascontiguousarray(P.transpose(0, 2, 1)); d2 = dYg.reshape(batch, cog, L); plan = _plan(batch * G, cog, K, L)
         dl = d2 if off is None else oracle.pam(d2, np.float32(off))
         assert_same_bits(dW_a[:, g * cog:(g + 1) * cog], oracle.gemm(dl, Pt, kchunk=plan), f"grouped weight gradient, group {g}")
         want = oracle.gemm(d2, Pt, mode=oracle.MODE_BWD_DELTA_L, D=np.broadcast_to(W2, (batch, cog, K)), offset=off, kchunk=plan)
@@ -236,7 +236,7 @@ def test_grouped_convolution_against_oracle(oracle, case, off):
             Pd = torch.nn.functional.unfold(torch.from_numpy(dYg), (kh, kw), padding=(kh - 1 - padding[0], kw - 1 - padding[1])).numpy()
             Kt = Pd.shape[1]
             Wf = np.ascontiguousarray(Wg.transpose(1, 0, 2, 3)[:, :, ::-1, ::-1]).reshape(cg, Kt)
-            plan = _plan(batch, cg, h * w, Kt)
+            plan = _plan(batch * G, cg, h * w, Kt)
             Wfl = Wf if off is None else oracle.pam(Wf, np.float32(off))
             assert_same_bits(dX_a[:, g * cg:(g + 1) * cg].reshape(batch, cg, h * w), oracle.gemm(np.broadcast_to(Wfl, (batch, cg, Kt)), Pd, kchunk=plan),
                              f"grouped input gradient, group {g}")
