@@ -199,7 +199,8 @@ int pam_hip_layer_norm_bwd(const float *x, const float *weight, const float *dy,
  * pam.conv2d_group (:163-198): w[co][c / groups][kh][kw], channels and filters fall into groups that
  * do not mix (groups = 1 otherwise); one launch covers all (image, group) pairs, with one copy of the
  * weights per image in the workspace where a product reads them -- unless those copies would exceed
- * 32 MiB, then one launch per group.  Sums run over k = (c, i, j) of the group in ascending order in
+ * 32 MiB, then one launch per group; depthwise convolutions (groups = c = co, kh*kw < 128) have kernels
+ * of their own that give the same sums in the same order.  Sums run over k = (c, i, j) of the group in ascending order in
  * the chunks pam_hip_gemm_plan(batch * groups, co / groups, ho*wo, (c / groups)*kh*kw) reports
  * (batch in place of batch * groups for a product that is launched per group). */
 size_t pam_hip_conv2d_workspace_bytes(long batch, long c, long h, long w, long co, long kh, long kw,

@@ -192,6 +192,9 @@ GROUPED = [
     (2, 8, 9, 8, 12, 3, 3, (1, 1), (1, 1), 4),
     (3, 6, 12, 10, 140, 3, 5, (2, 1), (0, 2), 2),        # 70 filters per group: more than one row tile
     (2, 16, 7, 7, 16, 3, 3, (1, 1), (1, 1), 16),         # depthwise
+    (3, 8, 12, 10, 8, 3, 5, (2, 1), (0, 2), 8),          # depthwise, strided, a 3 x 5 kernel
+    (1, 4, 40, 40, 4, 3, 3, (1, 1), (1, 1), 4),          # depthwise with few channels: the weight gradient's sum over 1600 positions is cut
+    (2, 6, 9, 9, 6, 5, 5, (1, 1), (4, 4), 6),            # depthwise, padding = kernel - 1
 ]
 
 
