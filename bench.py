@@ -363,6 +363,18 @@ def main():
                     other[f"{tag}_input_gradient_{kind}"] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1),
                                                             "valu_frac": round(ops * cm / (ms * 1e-3) / lane_peak, 4)}
             del gy, xc, wc
+        # grouped convolutions (one launch over (image, group) pairs) and a depthwise one (kernels of its own)
+        for tag, (cb, cc, chh, gr) in {"conv3x3_32x128x28x28_to128_groups32": (32, 128, 28, 32),
+                                       "conv3x3_32x192x28x28_depthwise": (32, 192, 28, 192)}.items():
+            xc = torch.randn(cb, cc, chh, chh, generator=g).to(dev); wc = (torch.randn(cc, cc // gr, 3, 3, generator=g) * 0.05).to(dev)
+            gy = (torch.randn(cb, cc, chh, chh, generator=g) * 1e-2).to(dev)
+            cm = cb * cc * chh * chh * (cc // gr) * 9
+            for name, fn in (("", lambda: abi.conv2d_fwd(xc, wc, (1, 1), (1, 1), 1.0, gr)),
+                             ("_weight_gradient_approx", lambda: abi.conv2d_bwd_weight(xc, gy, wc, (1, 1), (1, 1), False, 1.0, gr)),
+                             ("_input_gradient_approx", lambda: abi.conv2d_bwd_input(gy, wc, xc, (1, 1), False, 1.0, gr))):
+                ms = event_time_ms(fn, 30, torch)
+                other[tag + name] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1), "valu_frac": round(2 * cm / (ms * 1e-3) / lane_peak, 4)}
+            del gy, xc, wc
         na = 1 << 26
         pa, ga, ma, va = (torch.randn(na, generator=g).to(dev) * s_ for s_ in (1.0, 1e-2, 1e-2, 1e-4))
         va.abs_()

@@ -195,6 +195,7 @@ GROUPED = [
     (3, 8, 12, 10, 8, 3, 5, (2, 1), (0, 2), 8),          # depthwise, strided, a 3 x 5 kernel
     (1, 4, 40, 40, 4, 3, 3, (1, 1), (1, 1), 4),          # depthwise with few channels: the weight gradient's sum over 1600 positions is cut
     (2, 6, 9, 9, 6, 5, 5, (1, 1), (4, 4), 6),            # depthwise, padding = kernel - 1
+    (2, 4, 10, 9, 12, 3, 3, (1, 1), (1, 1), 4),          # one channel, three filters per group
 ]
 
 
