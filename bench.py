@@ -374,6 +374,8 @@ def main():
                              ("_input_gradient_approx", lambda: abi.conv2d_bwd_input(gy, wc, xc, (1, 1), False, 1.0, gr))):
                 ms = event_time_ms(fn, 30, torch)
                 other[tag + name] = {"ms": round(ms, 4), "gmacs": round(cm / ms / 1e6, 1), "valu_frac": round(2 * cm / (ms * 1e-3) / lane_peak, 4)}
+                if gr == cc:            # nine products per output: bound by the two tensors' bytes, if by anything
+                    other[tag + name]["hbm_frac"] = round(8 * xc.numel() / ms / 1e6 / 8000.0, 3)
             del gy, xc, wc
         na = 1 << 26
         pa, ga, ma, va = (torch.randn(na, generator=g).to(dev) * s_ for s_ in (1.0, 1e-2, 1e-2, 1e-4))
