@@ -15,8 +15,8 @@ import tempfile
 
 HERE = pathlib.Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
-SOURCES = sorted(CSRC.glob("pam_gemm_inst_*.hip")) + [CSRC / "pam_rowops.hip", CSRC / "pam_gemm.hip", CSRC / "pam_elementwise.hip",
-                                                      CSRC / "pam_probe.hip"]   # slowest first
+SOURCES = [CSRC / "pam_rowops_plain.hip", CSRC / "pam_rowops_offset.hip"] + sorted(CSRC.glob("pam_gemm_inst_*.hip")) + [
+    CSRC / "pam_gemm.hip", CSRC / "pam_elementwise.hip", CSRC / "pam_rowops.hip", CSRC / "pam_probe.hip"]   # slowest first
 JOBS = 8
 STAMP_SOURCE = CSRC / "pam_stamp.cpp"
 LIB = HERE / "lib" / "libpam_hip.so"
