@@ -417,30 +417,47 @@ struct DirectGeom { int IC, H, W, ho, wo, kh, kw, sh, sw, ph, pw, gin, gout; };
 // upstream gradient, the stride-1 geometry of that convolution, the sum over a group's filters).
 // EXACT false: term = (weight (*) off) (*) v -- the forward and the approximate input gradient; EXACT true:
 // term = pam_bwd(d, weight, v) with the offset on the weight, d = the output position's own forward input.
-template <bool EXACT>
+// SIDE: the kernel is SIDE x SIDE taps and the loops over them are unrolled (all of a channel's loads in flight
+// together); 0: any kernel size.
+template <bool EXACT, int SIDE>
 __global__ __launch_bounds__(256) void direct_conv_kernel(const float* __restrict__ img, const float* __restrict__ w, const float* __restrict__ d,
                                                          float* __restrict__ out, long total, int planes, DirectGeom q, int transposed, float off,
                                                          int has_off)
 {
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
-    const int ow = (int)(idx % q.wo), oh = (int)((idx / q.wo) % q.ho);
-    const long plane = idx / ((long)q.wo * q.ho);                         // b * planes + p
-    const int p = (int)(plane % planes), g = p / q.gout, oc = p % q.gout, taps = q.kh * q.kw;
-    const long b = plane / planes;
+    int ow, oh, p; long b;                                                // idx = ((b planes + p) ho + oh) wo + ow
+    if (total <= 0x7fffffffL) {                                           // (32-bit divisions where they do: the 64-bit ones are long)
+        const int at = (int)idx, hw = q.wo * q.ho, plane = at / hw, l = at - plane * hw, b32 = plane / planes;
+        oh = l / q.wo; ow = l - oh * q.wo; p = plane - b32 * planes; b = b32;
+    } else {
+        const long plane = idx / ((long)q.wo * q.ho);
+        ow = (int)(idx % q.wo); oh = (int)((idx / q.wo) % q.ho); p = (int)(plane % planes); b = plane / planes;
+    }
+    const int kh = SIDE ? SIDE : q.kh, kw = SIDE ? SIDE : q.kw;
+    const int g = p / q.gout, oc = p % q.gout, taps = kh * kw;
     const float dv = EXACT ? d[idx] : 0.0f;
     float acc = 0.0f;
     for (int c = 0; c < q.gin; ++c) {
         const float* base = img + (b * q.IC + g * q.gin + c) * (long)q.H * q.W;
         const float* wc = w + (transposed ? ((long)(g * q.gin + c) * q.gout + oc) : ((long)p * q.gin + c)) * taps;
-        for (int i = 0; i < q.kh; ++i) {
+#pragma unroll
+        for (int i = 0; i < kh; ++i) {
             const int h = oh * q.sh - q.ph + i;
-            for (int j = 0; j < q.kw; ++j) {
-                const int x = ow * q.sw - q.pw + j, k = i * q.kw + j;
+#pragma unroll
+            for (int j = 0; j < kw; ++j) {
+                const int x = ow * q.sw - q.pw + j, k = i * kw + j;
                 const float wk = wc[transposed ? taps - 1 - k : k];
                 const bool inside = (unsigned)h < (unsigned)q.H && (unsigned)x < (unsigned)q.W;
                 const float v = inside ? base[(long)h * q.W + x] : 0.0f;
-                acc = acc + (EXACT ? pam_mul_bwd(dv, wk, v, off, has_off != 0) : pam_mul(has_off ? pam_mul(wk, off) : wk, v));
+                // A padding position's term is a zero, and adding it changes nothing (the sum starts at +0 and never
+                // becomes -0) -- unless the weight (or d) is inf or NaN, which makes the term NaN: only then is it
+                // computed.  (Computed always, the zeros took the primitives' full definition in nearly every wavefront.)
+                const float ws = has_off ? pam_mul(wk, off) : wk;              // (the weight as the product sees it)
+                // (EXACT: the slope of a weight of 2^127 and more can be inf, and inf times the zero NaN)
+                const bool finite = (f2u(ws) & 0x7fffffffu) < (EXACT ? 0x7f000000u : 0x7f800000u) && (!EXACT || (f2u(dv) & 0x7f800000u) != 0x7f800000u);
+                if (inside || !finite)
+                    acc = acc + (EXACT ? pam_mul_bwd(dv, wk, v, off, has_off != 0) : pam_mul(ws, v));
             }
         }
     }
@@ -458,8 +475,9 @@ __global__ __launch_bounds__(256) void direct_conv_weight_kernel(const float* __
 {
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
-    const int taps = q.kh * q.kw, K = q.gin * taps, k = (int)(idx % K), c = k / taps, i = (k % taps) / q.kw, j = k % q.kw;
-    const long plane = idx / K;                                            // b * filters + co
+    const int taps = q.kh * q.kw, K = q.gin * taps;
+    const long plane = total <= 0x7fffffffL ? (long)((int)idx / K) : idx / K;          // b * filters + co
+    const int k = (int)(idx - plane * K), c = k / taps, i = (k % taps) / q.kw, j = k % q.kw;
     const int co = (int)(plane % filters), L = q.ho * q.wo;
     const long b = plane / filters;
     const float* base = x + (b * q.IC + (co / q.gout) * q.gin + c) * (long)q.H * q.W;
@@ -473,11 +491,26 @@ __global__ __launch_bounds__(256) void direct_conv_weight_kernel(const float* __
             const int h = (l / q.wo) * q.sh - q.ph + i, xx = (l % q.wo) * q.sw - q.pw + j;
             const bool inside = (unsigned)h < (unsigned)q.H && (unsigned)xx < (unsigned)q.W;
             const float v = inside ? base[(long)h * q.W + xx] : 0.0f, gl = g[l];
-            part = part + (EXACT ? pam_mul_bwd(wk, v, gl, off, has_off != 0) : pam_mul(has_off ? pam_mul(gl, off) : gl, v));
+            // (a padding position's term is a zero unless the gradient -- or w -- is inf or NaN: see direct_conv_kernel)
+            const float gs = !EXACT && has_off ? pam_mul(gl, off) : gl;         // (the gradient as the approximate product sees it)
+            const bool finite = (f2u(gs) & 0x7f800000u) != 0x7f800000u && (!EXACT || (f2u(wk) & 0x7f800000u) != 0x7f800000u);
+            if (inside || !finite)
+                part = part + (EXACT ? pam_mul_bwd(wk, v, gl, off, has_off != 0) : pam_mul(gs, v));
         }
         sum = chunk >= L ? part : sum + part;
     }
     dw[idx] = sum;
+}
+
+template <bool EXACT>
+void launch_direct_conv(const float* img, const float* w, const float* d, float* out, long total, int planes, const DirectGeom& q,
+                        int transposed, float off, hipStream_t st)
+{
+    const dim3 grid((unsigned)((total + 255) / 256));
+    const int has_off = off != 1.0f ? 1 : 0, side = q.kh == q.kw ? q.kh : 0;
+#define PAM_DIRECT_SIDE(S) hipLaunchKernelGGL((direct_conv_kernel<EXACT, S>), grid, dim3(256), 0, st, img, w, d, out, total, planes, q, transposed, off, has_off)
+    if (side == 3) PAM_DIRECT_SIDE(3); else if (side == 5) PAM_DIRECT_SIDE(5); else if (side == 7) PAM_DIRECT_SIDE(7); else PAM_DIRECT_SIDE(0);
+#undef PAM_DIRECT_SIDE
 }
 
 // Which grouped convolutions: groups of up to kDirectGroup channels and filters whose sums (either way round) are short
@@ -648,10 +681,9 @@ int pam_hip_conv2d_bwd_input(const float* dy, const float* w, const float* x, fl
     if (direct_conv(s)) {                             // the convolution of dy with the flipped weights, directly
         const long total = batch * c * h * wd;
         if (total >= (1L << 31) * 256) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_bwd_input: too many outputs");
-        const dim3 grid((unsigned)((total + 255) / 256));
         const DirectGeom q = direct_geom(t);          // (t: the image is dy, a group's sums run over its filters)
-        if (exact) hipLaunchKernelGGL(direct_conv_kernel<true>, grid, dim3(256), 0, st, dy, w, x, dx, total, (int)c, q, 1, offset, offset != 1.0f ? 1 : 0);
-        else hipLaunchKernelGGL(direct_conv_kernel<false>, grid, dim3(256), 0, st, dy, w, (const float*)nullptr, dx, total, (int)c, q, 1, offset, offset != 1.0f ? 1 : 0);
+        if (exact) launch_direct_conv<true>(dy, w, x, dx, total, (int)c, q, 1, offset, st);
+        else launch_direct_conv<false>(dy, w, nullptr, dx, total, (int)c, q, 1, offset, st);
         return pamhost::check_launch("conv2d_bwd_input");
     }
     ConvSpace sp = input_gradient_space(t);
@@ -704,8 +736,7 @@ int pam_hip_conv2d_fwd(const float* x, const float* w, float* y, long batch, lon
     if (direct_conv(s)) {
         const long total = batch * co * s.L();
         if (total >= (1L << 31) * 256) return pamhost::fail(PAM_HIP_ERR_ARGUMENT, "conv2d_fwd: too many outputs");
-        hipLaunchKernelGGL(direct_conv_kernel<false>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, x, w, (const float*)nullptr, y, total,
-                           (int)co, direct_geom(s), 0, offset, has_off ? 1 : 0);
+        launch_direct_conv<false>(x, w, nullptr, y, total, (int)co, direct_geom(s), 0, offset, st);
         return pamhost::check_launch("conv2d_fwd");
     }
     ConvSpace sp = conv_space(s, 0, has_off);

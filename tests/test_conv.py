@@ -206,16 +206,30 @@ def test_grouped_convolution_against_oracle(oracle, case, off):
     stride 1, both input gradients against the oracle's products on the unfolded slices."""
     batch, c, h, w, co, kh, kw, stride, padding, G = case
     cg, cog = c // G, co // G
+    _grouped_case(oracle, case, off, odd_weights=False)
+    if G == c == co:
+        # depthwise kernels leave out the terms of padding positions, which are zeros -- unless a weight or an upstream
+        # gradient is inf or NaN (or becomes inf with the offset): then the term is NaN, as in the matrix kernel
+        _grouped_case(oracle, case, off, odd_weights=True)
+
+
+def _grouped_case(oracle, case, off, odd_weights):
+    batch, c, h, w, co, kh, kw, stride, padding, G = case
+    cg, cog = c // G, co // G
     rng = np.random.RandomState(11)
     X = rng.standard_normal((batch, c, h, w)).astype(np.float32)
     W = (rng.standard_normal((co, cg, kh, kw)) * 0.1).astype(np.float32)
     X.reshape(-1)[rng.choice(X.size, 5, replace=False)] = [0.0, -0.0, 1e-40, -3e38, 7.0]
+    if odd_weights:
+        W.reshape(-1)[rng.choice(W.size, 4, replace=False)] = [np.inf, np.nan, 3.3e38, 0.0]
     o = 1.0 if off is None else off
     Xd, Wd = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda()
     Y = _abi.conv2d_fwd(Xd, Wd, stride, padding, o, G)
     ho, wo = Y.shape[2:]
     L = ho * wo
     dY = (rng.standard_normal((batch, co, ho, wo)) * 1e-2).astype(np.float32)
+    if odd_weights:
+        dY.reshape(-1)[rng.choice(dY.size, 4, replace=False)] = [np.inf, np.nan, -3.3e38, 0.0]
     dYd = torch.from_numpy(dY).cuda()
     dW_a = _abi.conv2d_bwd_weight(Xd, dYd, Wd, stride, padding, False, o, G).cpu().numpy()
     dW_e = _abi.conv2d_bwd_weight(Xd, dYd, Wd, stride, padding, True, o, G).cpu().numpy()
