@@ -35,6 +35,8 @@ def _inputs(case, seed, specials=False):
     if specials:
         flat = X.reshape(-1)
         flat[rng.choice(flat.size, 6, replace=False)] = [0.0, -0.0, 1e-40, -3e38, np.inf, np.nan]
+        # (and weights whose products with a padding zero are not zeros: inf, NaN, and 2^127 and more, whose slope is inf)
+        W.reshape(-1)[rng.choice(W.size, 5, replace=False)] = [np.inf, np.nan, 3.3e38, 0.0, -1e-40]
     return X, W
 
 
