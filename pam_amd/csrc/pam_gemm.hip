@@ -487,15 +487,28 @@ __global__ __launch_bounds__(256) void direct_conv_weight_kernel(const float* __
     for (int l0 = 0; l0 < L; l0 += chunk) {
         float part = 0.0f;
         const int end = min(L, l0 + chunk);
-        for (int l = l0; l < end; ++l) {
-            const int h = (l / q.wo) * q.sh - q.ph + i, xx = (l % q.wo) * q.sw - q.pw + j;
-            const bool inside = (unsigned)h < (unsigned)q.H && (unsigned)xx < (unsigned)q.W;
-            const float v = inside ? base[(long)h * q.W + xx] : 0.0f, gl = g[l];
-            // (a padding position's term is a zero unless the gradient -- or w -- is inf or NaN: see direct_conv_kernel)
-            const float gs = !EXACT && has_off ? pam_mul(gl, off) : gl;         // (the gradient as the approximate product sees it)
-            const bool finite = (f2u(gs) & 0x7f800000u) != 0x7f800000u && (!EXACT || (f2u(wk) & 0x7f800000u) != 0x7f800000u);
-            if (inside || !finite)
-                part = part + (EXACT ? pam_mul_bwd(wk, v, gl, off, has_off != 0) : pam_mul(gs, v));
+        // eight positions' loads in flight at a time (there are few lanes, each with a long chain of sums); the terms
+        // are added one by one in ascending order all the same
+        constexpr int kAhead = 8;
+        for (int lb = l0; lb < end; lb += kAhead) {
+            float v[kAhead], gv[kAhead]; bool in[kAhead];
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                const int l = min(lb + u, end - 1);
+                const int h = (l / q.wo) * q.sh - q.ph + i, xx = (l % q.wo) * q.sw - q.pw + j;
+                in[u] = (unsigned)h < (unsigned)q.H && (unsigned)xx < (unsigned)q.W;
+                v[u] = in[u] ? base[(long)h * q.W + xx] : 0.0f; gv[u] = g[l];
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                if (lb + u >= end) break;
+                const float gl = gv[u];
+                // (a padding position's term is a zero unless the gradient -- or w -- is inf or NaN: see direct_conv_kernel)
+                const float gs = !EXACT && has_off ? pam_mul(gl, off) : gl;     // (the gradient as the approximate product sees it)
+                const bool finite = (f2u(gs) & 0x7f800000u) != 0x7f800000u && (!EXACT || (f2u(wk) & 0x7f800000u) != 0x7f800000u);
+                if (in[u] || !finite)
+                    part = part + (EXACT ? pam_mul_bwd(wk, v[u], gl, off, has_off != 0) : pam_mul(gs, v[u]));
+            }
         }
         sum = chunk >= L ? part : sum + part;
     }
