@@ -1182,18 +1182,16 @@ __global__ __launch_bounds__((BM / TM) * (BN / TN)) PAM_GEMM_OCCUPANCY void gemm
             u32x4 fa0 = *reinterpret_cast<LdsVec>(pl), fb0 = *reinterpret_cast<LdsVec>(pr), fa1, fb1;
 #pragma unroll 1
             for (int kk = 0; kk < BK; kk += 4) {
-                pl += LDL * 4; pr += LDR * 4;
-                fa1 = *reinterpret_cast<LdsVec>(pl); fb1 = *reinterpret_cast<LdsVec>(pr);
+                // (the reads of a four at constant distances from one address: one address update per operand and four)
+                fa1 = *reinterpret_cast<LdsVec>(pl + LDL * 4); fb1 = *reinterpret_cast<LdsVec>(pr + LDR * 4);
                 step(kk, fa0, fb0);
-                pl += LDL * 4; pr += LDR * 4;
-                fa0 = *reinterpret_cast<LdsVec>(pl); fb0 = *reinterpret_cast<LdsVec>(pr);
+                fa0 = *reinterpret_cast<LdsVec>(pl + 2 * LDL * 4); fb0 = *reinterpret_cast<LdsVec>(pr + 2 * LDR * 4);
                 step(kk + 1, fa1, fb1);
-                pl += LDL * 4; pr += LDR * 4;
-                fa1 = *reinterpret_cast<LdsVec>(pl); fb1 = *reinterpret_cast<LdsVec>(pr);
+                fa1 = *reinterpret_cast<LdsVec>(pl + 3 * LDL * 4); fb1 = *reinterpret_cast<LdsVec>(pr + 3 * LDR * 4);
                 step(kk + 2, fa0, fb0);
                 // (the last four read their own last step again: a read under a condition would make the wait before
                 // the block below one for all reads, the two just issued included)
-                pl += kk + 4 < BK ? LDL * 4 : 0; pr += kk + 4 < BK ? LDR * 4 : 0;
+                pl += (kk + 4 < BK ? 4 : 3) * LDL * 4; pr += (kk + 4 < BK ? 4 : 3) * LDR * 4;
                 if (BK == 32 && kk == 12) { pl += to_plx; pr += to_prx; }        // (see swizzled)
                 fa0 = *reinterpret_cast<LdsVec>(pl); fb0 = *reinterpret_cast<LdsVec>(pr);
                 step(kk + 3, fa1, fb1);
