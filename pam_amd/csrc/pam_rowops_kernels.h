@@ -878,6 +878,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
 // GradUncheckedT is the all-approximate chain on the branch-free primitives, tried first and kept
 // when every value it touched was a normal number.
 struct GradChecked {
+    static constexpr bool kOffsets = true, kApproxUnchecked = false;
     Offset o; Approx ap;
     __device__ __forceinline__ float mul(float a, float b) { return pam_mul_off(a, b, o.off, o.has); }
     __device__ __forceinline__ float div(float a, float b) { return pad_div_off(a, b, o.off, o.has); }
@@ -910,6 +911,7 @@ __device__ __forceinline__ float log2_exact_dx_unchecked(float x, float g, Span&
 }
 template <bool OFFSETS>
 struct GradUncheckedT {
+    static constexpr bool kOffsets = OFFSETS, kApproxUnchecked = true;
     Offset o; Span sp;
     __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked_off(a, b, o.off, OFFSETS && o.has, sp); }
     __device__ __forceinline__ float div(float a, float b) { return pad_unchecked_off(a, b, o.off, OFFSETS && o.has, sp); }
@@ -935,6 +937,7 @@ template <RowKernel K, int CH, bool BLOCK> using GradUncheckedFor = GradUnchecke
 // 2^e(exp2 x) g; of log2, 2^-e(x) g.  The products with the upstream gradients are IEEE products in the checked forms
 // too, so the gradients need no recording; the other operands are recorded, with the extra headroom the carries need.
 struct GradUncheckedExact {
+    static constexpr bool kOffsets = false, kApproxUnchecked = false;
     Offset o; Span sp;                            // used without an offset only
     __device__ __forceinline__ float mul(float a, float b) { return pam_unchecked(a, b, sp); }
     __device__ __forceinline__ float div(float a, float b) { return pad_unchecked(a, b, sp); }
@@ -1091,12 +1094,70 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(PAM_RO
     }
 }
 
+// Which instances of the layer_norm gradient take the cheaper forms (see layer_norm_grad_row): by measurement.
+template <int CH, class L>
+constexpr bool layer_norm_grad_cheap() { return true; }
+
 // One row of the layer_norm gradient.  cen: x on entry, overwritten; g: dy on entry (1.0 past the
 // end), dx on exit; terms: the per-element terms of the weight gradient (if weight).
 template <int CH, class G, class L, class P>
 __device__ __forceinline__ void layer_norm_grad_row(float (&cen)[CH], float (&g)[CH], float (&terms)[CH],
                                                     const P& par, L& lay, long n, float count, float eps, G& m)
 {
+    // The all-approximate chain without an offset, on the cheaper forms of the unchecked primitives where an operand is
+    // the row's positive denominator (recorded once), a value the chain has recorded already, or the same product twice:
+    // the same bits, fewer magnitudes to record and fewer products.  In the instances where that measured faster.
+    if constexpr (G::kApproxUnchecked && !G::kOffsets && layer_norm_grad_cheap<CH, L>()) {
+        float p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) p = p + cen[c];
+        const float s1 = lay.sum(p);
+        const float mu = m.div(s1, count);
+        p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) { cen[c] = cen[c] - mu; const float sq = pam_unchecked_square(cen[c], m.sp); if (lay.index(c) < n) p = p + sq; }
+        const float s2 = lay.sum(p);
+        const float v = m.div(s2, count) + eps;
+        const float lg = m.log2(v);
+        const float half = m.mul(lg, 0.5f);
+        const float root = m.exp2(half);
+        const float denom = v == 0.0f ? 0.0f : root;
+        m.sp.see(f2u(denom) & ~kSign);
+        const float inv = m.div(1.0f, denom);
+        p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const long i = lay.index(c); const bool inside = i < n;
+            const float xn = pad_unchecked_by_positive(cen[c], denom, m.sp);           // (the centred value was recorded by its square)
+            if (par.weight) {
+                const float wi = par.weight_at(c, i, inside);
+                terms[c] = pam_unchecked_seen(xn, g[c], m.sp);
+                g[c] = m.mul(g[c], wi);
+            }
+            const float d = -pam_unchecked_seen(pad_unchecked_by_positive(xn, denom, m.sp), g[c], m.sp);
+            if (inside) p = p + d;
+        }
+        float d = lay.sum(p);
+        if (v == 0.0f) d = 0.0f;
+        d = m.exp2_dx(half, d);
+        d = m.mul_da(lg, 0.5f, d);
+        d = m.log2_dx(v, d);
+        const float ds2 = m.div_da(s2, count, d);
+        p = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float dc = pam_unchecked_seen(inv, g[c], m.sp);
+            const float t = pam_unchecked_seen(cen[c], ds2, m.sp);                      // both operands of c (*) c get this gradient
+            dc = dc + t;
+            dc = dc + t;
+            g[c] = dc;
+            if (lay.index(c) < n) p = p + dc;
+        }
+        const float ds1 = m.div_da(s1, count, -lay.sum(p));
+#pragma unroll
+        for (int c = 0; c < CH; ++c) g[c] = g[c] + ds1;
+        return;
+    }
     float p = 0.0f;
 #pragma unroll
     for (int c = 0; c < CH; ++c) p = p + cen[c];                        // the fill adds +0
