@@ -391,37 +391,39 @@ def test_gpu_softmax_special_values(oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n", [100, 150, 350, 700, 2000, 20000])
-def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n):
-    """All-exact gradients without an offset first run on unchecked arithmetic: inputs and upstream gradients at and
-    beyond the edges of what that accepts (zeros, subnormals, huge and tiny values, inf, NaN, a variance of exactly 1)."""
+@pytest.mark.parametrize("approx", [False, True])
+@pytest.mark.parametrize("n", [60, 100, 150, 200, 350, 512, 700, 1000, 2000, 20000])      # (every values-per-lane instance)
+def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n, approx):
+    """All-exact (and all-approximate) gradients without an offset first run on unchecked arithmetic: inputs and upstream
+    gradients at and beyond the edges of what that accepts (zeros, subnormals, huge and tiny values, inf, NaN, a variance
+    of exactly 1)."""
     rng = np.random.RandomState(n)
     x = (rng.standard_normal((12, n)) * 3).astype(np.float32)
     x[1, 3] = 0.0; x[2, 5] = 1e-40; x[3, 7] = 3e38; x[4, 9] = -3e38; x[5, 11] = 2.0 ** -120; x[6, :] = 2.0 ** 100; x[7, 13] = -np.inf
     x[8, :] = np.where(np.arange(n) % 2 == 0, 1.0, -1.0)             # mean 0, variance 1 (n even)
     g = rng.standard_normal(x.shape).astype(np.float32)
     g[0, 1] = 0.0; g[0, 2] = 1e-42; g[1, 4] = np.inf; g[2, 6] = np.nan; g[3, 8] = 3e38; g[9, :] = 0.0; g[10, 3] = 2.0 ** -130
-    flags = (False, False, False)
+    flags = (approx, approx, approx)
     xt = _dev(x).requires_grad_()
-    y = pam_amd.softmax(xt, dim=-1)
+    y = pam_amd.softmax(xt, dim=-1, approx_bwd=approx)
     want, row_sum, shift = oracle.softmax_fwd(x)
     assert_same_bits(y.detach().cpu().numpy(), want, "softmax")
     y.backward(_dev(g))
     assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, None, flags), "softmax gradient")
     xf = np.where(np.isfinite(x), x, np.float32(1.5)).astype(np.float32)
     xt = _dev(xf).requires_grad_()
-    y = pam_amd.log_softmax(xt, dim=-1)
+    y = pam_amd.log_softmax(xt, dim=-1, approx_bwd=approx)
     y.backward(_dev(g))
     sh = np.floor(oracle.pam(xf, C).max())
     assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g, sh, None, flags, log_softmax=True), "log_softmax gradient")
     xt = _dev(xf).requires_grad_()
-    pam_amd.logsumexp(xt, dim=-1).backward(_dev(g[:, 0].copy()))
+    pam_amd.logsumexp(xt, dim=-1, approx_bwd=approx).backward(_dev(g[:, 0].copy()))
     assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g[:, 0].copy(), sh, None, flags), "logsumexp gradient")
     w = (rng.standard_normal(n) + 2).astype(np.float32); w[3] = 0.0; w[5] = 1e-39; w[7] = -2.0
     for ww in (None, w):
         xt = _dev(xf).requires_grad_()
         wt = None if ww is None else _dev(ww).requires_grad_()
-        y = pam_amd.layer_norm(xt, n, wt, None)
+        y = pam_amd.layer_norm(xt, n, wt, None, approx_bwd=approx)
         y.backward(_dev(g))
         dx, _ = oracle.layer_norm_bwd(xf, ww, g, 1e-5, None, flags)
         assert_same_bits(xt.grad.cpu().numpy(), dx, "layer_norm gradient")
