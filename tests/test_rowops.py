@@ -391,9 +391,10 @@ def test_gpu_softmax_special_values(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("off", [None, OFF])
 @pytest.mark.parametrize("approx", [False, True])
 @pytest.mark.parametrize("n", [60, 100, 150, 200, 350, 512, 700, 1000, 2000, 20000])      # (every values-per-lane instance)
-def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n, approx):
+def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n, approx, off):
     """All-exact (and all-approximate) gradients without an offset first run on unchecked arithmetic: inputs and upstream
     gradients at and beyond the edges of what that accepts (zeros, subnormals, huge and tiny values, inf, NaN, a variance
     of exactly 1)."""
@@ -405,27 +406,27 @@ def test_gpu_exact_gradients_at_the_edges_of_the_unchecked_forms(oracle, n, appr
     g[0, 1] = 0.0; g[0, 2] = 1e-42; g[1, 4] = np.inf; g[2, 6] = np.nan; g[3, 8] = 3e38; g[9, :] = 0.0; g[10, 3] = 2.0 ** -130
     flags = (approx, approx, approx)
     xt = _dev(x).requires_grad_()
-    y = pam_amd.softmax(xt, dim=-1, approx_bwd=approx)
-    want, row_sum, shift = oracle.softmax_fwd(x)
+    y = pam_amd.softmax(xt, dim=-1, approx_bwd=approx, offset=off)
+    want, row_sum, shift = oracle.softmax_fwd(x, off)
     assert_same_bits(y.detach().cpu().numpy(), want, "softmax")
     y.backward(_dev(g))
-    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, None, flags), "softmax gradient")
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.softmax_bwd(x, g, row_sum, shift, off, flags), "softmax gradient")
     xf = np.where(np.isfinite(x), x, np.float32(1.5)).astype(np.float32)
     xt = _dev(xf).requires_grad_()
-    y = pam_amd.log_softmax(xt, dim=-1, approx_bwd=approx)
+    y = pam_amd.log_softmax(xt, dim=-1, approx_bwd=approx, offset=off)
     y.backward(_dev(g))
-    sh = np.floor(oracle.pam(xf, C).max())
-    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g, sh, None, flags, log_softmax=True), "log_softmax gradient")
+    sh = np.floor(oracle.pam(xf, C, off).max())
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g, sh, off, flags, log_softmax=True), "log_softmax gradient")
     xt = _dev(xf).requires_grad_()
-    pam_amd.logsumexp(xt, dim=-1, approx_bwd=approx).backward(_dev(g[:, 0].copy()))
-    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g[:, 0].copy(), sh, None, flags), "logsumexp gradient")
+    pam_amd.logsumexp(xt, dim=-1, approx_bwd=approx, offset=off).backward(_dev(g[:, 0].copy()))
+    assert_same_bits(xt.grad.cpu().numpy(), oracle.logsumexp_bwd(xf, g[:, 0].copy(), sh, off, flags), "logsumexp gradient")
     w = (rng.standard_normal(n) + 2).astype(np.float32); w[3] = 0.0; w[5] = 1e-39; w[7] = -2.0
     for ww in (None, w):
         xt = _dev(xf).requires_grad_()
         wt = None if ww is None else _dev(ww).requires_grad_()
-        y = pam_amd.layer_norm(xt, n, wt, None, approx_bwd=approx)
+        y = pam_amd.layer_norm(xt, n, wt, None, approx_bwd=approx, offset=off)
         y.backward(_dev(g))
-        dx, _ = oracle.layer_norm_bwd(xf, ww, g, 1e-5, None, flags)
+        dx, _ = oracle.layer_norm_bwd(xf, ww, g, 1e-5, off, flags)
         assert_same_bits(xt.grad.cpu().numpy(), dx, "layer_norm gradient")
 
 
